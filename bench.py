@@ -1,0 +1,232 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused-MoE forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME] [--split 0|1] [--all]
+
+A "step" is one call of the fused op over one batch of synthetic input that is already
+resident in HBM (routing, moe_align and quantisation happen before the timed region, as in the
+reference's benchmark/benchmark.py:19-22).  The default workload is the Mixtral-8x7B-like bf16
+prefill shape with split=True.  The last line printed is one JSON object: whole-op throughput
+(`value`), the roofline figure of the dominant kernel measured with HIP events in this run, and
+the CPU oracle timed on the host cores on a bounded sample of the same workload.
+
+`--all` additionally prints one line per benchmark configuration (time, TFLOP/s, GB/s, % of
+roofline) to stderr.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "prime-flash-moe_amd"))
+sys.path.insert(0, ROOT)
+
+import torch  # noqa: E402
+
+# MI355X published dense peaks
+PEAK_TFLOPS = {"bf16": 2500.0, "mxfp8": 5000.0}
+PEAK_HBM_GBS = 8000.0
+
+PHASE_ZERO, PHASE_UP, PHASE_DOWN, PHASE_FINALIZE, PHASE_ALL = 1, 2, 4, 8, 15
+
+
+def build_case(cfg, device, seed=0):
+    import prime_moe  # noqa: F401
+    from prime_moe.workloads import make_inputs
+    inp = make_inputs(cfg, device, seed=seed)
+    sched = torch.ops.prime_moe.moe_align(inp["topk_ids"], cfg.E, cfg.block_m, 1)
+    out = torch.zeros((cfg.T, cfg.K), dtype=torch.bfloat16, device=device)
+    return inp, sched, out
+
+
+def make_step(cfg, inp, sched, out, split):
+    import prime_moe
+    if cfg.dtype == "bf16":
+        def op():
+            prime_moe.fused_moe_bf16(inp["x"], inp["w1"], inp["w2"], *sched, inp["topk_weights"], out,
+                                     cfg.top_k, cfg.block_m, 64, 4, 2, 1, 1, split)
+    else:
+        def op():
+            prime_moe.fused_moe_mxfp8(inp["x"], inp["x_scales"], inp["w1"], inp["w1_scales"], inp["w2"],
+                                      inp["w2_scales"], *sched, inp["topk_weights"], out, cfg.top_k,
+                                      cfg.block_m, 64, 4, 2, 1, split)
+    if split:
+        return op
+
+    def step():  # the fused pipeline accumulates into `out`: zeroing it is part of the step
+        out.zero_()
+        op()
+    return step
+
+
+def time_steps(step, steps, warmup):
+    """Wall clock over exactly `steps` calls, synchronised on both sides; returns seconds/step."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def time_events(step, steps):
+    """Average duration of `step` from HIP events recorded on the stream the kernels run on."""
+    start = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stop = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    for i in range(steps):
+        start[i].record()
+        step()
+        stop[i].record()
+    torch.cuda.synchronize()
+    ms = sorted(s.elapsed_time(e) for s, e in zip(start, stop))
+    return sum(ms) / len(ms) * 1e-3, ms[len(ms) // 2] * 1e-3
+
+
+def phase_time(step, mask, steps):
+    from prime_moe import _native
+    lib = _native.load()
+    lib.pmoe_set_phase_mask(mask)
+    try:
+        for _ in range(2):
+            step()
+        return time_events(step, steps)[0]
+    finally:
+        lib.pmoe_set_phase_mask(PHASE_ALL)
+
+
+def hbm_bytes(cfg, inp):
+    """Algorithmic bytes of one call: weights (+scales) of the touched experts, x, out, routing."""
+    from prime_moe.workloads import touched_weight_bytes
+    wb = touched_weight_bytes(cfg, inp["topk_ids"])
+    xb = cfg.T * cfg.K * (2 if cfg.dtype == "bf16" else 1 + 1 / 32)
+    return wb, int(wb + xb + cfg.T * cfg.K * 2 + cfg.T * cfg.top_k * 8)
+
+
+def cpu_baseline(cfg, inp, gpu_out, budget_tokens):
+    """The CPU oracle (fp32 torch on the host cores) on the first `budget_tokens` tokens."""
+    from oracle import moe_oracle as O
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    n = min(cfg.T, budget_tokens)
+    ids = inp["topk_ids"][:n].cpu()
+    wts = inp["topk_weights"][:n].cpu()
+    if cfg.dtype == "bf16":
+        x, w1, w2 = inp["x"][:n].cpu(), inp["w1"].cpu(), inp["w2"].cpu()
+        run = lambda: O.fused_moe_dense(x, w1, w2, ids, wts)
+    else:
+        raise NotImplementedError("cpu baseline for mxfp8 is timed through tests/bench --all on bf16 only")
+    run()  # warm-up (thread pool, page faults)
+    t0 = time.perf_counter()
+    ref = run()
+    dt = time.perf_counter() - t0
+    flops = 3.0 * n * cfg.top_k * cfg.K * cfg.N
+    err = None
+    if gpu_out is not None:
+        got = gpu_out[:n].float().cpu()
+        err = float(((got - ref).abs() / ref.abs().clamp_min(1.0)).max())
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"first {n} of {cfg.T} tokens through all {cfg.E} experts, fp32 torch oracle, {dt:.2f} s"}, err
+
+
+def run_config(cfg, split, steps, warmup, device, with_cpu, log):
+    inp, sched, out = build_case(cfg, device)
+    step = make_step(cfg, inp, sched, out, split)
+    sec = time_steps(step, steps, warmup)
+    ev_mean, ev_med = time_events(step, steps)
+    t_up = phase_time(step, PHASE_UP, steps)
+    t_down = phase_time(step, PHASE_DOWN, steps) if split else 0.0
+    step()
+    torch.cuda.synchronize()
+    P = cfg.T * cfg.top_k
+    flops_up = 2.0 * P * cfg.K * cfg.N
+    flops_down = 1.0 * P * cfg.K * cfg.N
+    wb, total_b = hbm_bytes(cfg, inp)
+    peak = PEAK_TFLOPS[cfg.dtype]
+    res = {
+        "name": cfg.name, "split": bool(split), "sec": sec, "ev_mean": ev_mean, "ev_med": ev_med,
+        "t_up": t_up, "t_down": t_down, "tflops": cfg.flops / sec / 1e12,
+        "pct_mfma": 100 * cfg.flops / sec / 1e12 / peak, "weight_gbs": wb / sec / 1e9,
+        "pct_hbm": 100 * total_b / sec / 1e9 / PEAK_HBM_GBS, "weight_bytes": wb, "bytes": total_b,
+        "up_tflops": flops_up / t_up / 1e12 if t_up else 0.0,
+        "down_tflops": flops_down / t_down / 1e12 if t_down else 0.0,
+    }
+    log(f"{cfg.name:18s} split={int(split)}  {sec * 1e6:10.1f} us/call  {res['tflops']:8.1f} TFLOP/s "
+        f"({res['pct_mfma']:5.1f}% {cfg.dtype} MFMA peak)  weights {res['weight_gbs']:7.1f} GB/s  "
+        f"all-bytes {res['pct_hbm']:5.1f}% of 8 TB/s | up {t_up * 1e6:9.1f} us ({res['up_tflops']:7.1f} TF) "
+        f"down {t_down * 1e6:9.1f} us ({res['down_tflops']:7.1f} TF)")
+    cpu, err = (None, None)
+    if with_cpu:
+        cpu, err = cpu_baseline(cfg, inp, out, budget_tokens=512)
+        log(f"  cpu oracle: {cpu['value']:.3f} TFLOP/s on {cpu['cores']} cores ({cpu['sample']}); "
+            f"GPU vs oracle rel_clamp_1 = {err:.3g}")
+    res["cpu"], res["parity"] = cpu, err
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="c2_mixtral_bf16")
+    ap.add_argument("--split", type=int, default=1)
+    ap.add_argument("--all", action="store_true", help="also time every benchmark configuration (stderr)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path is single-device, "
+                 "there is no collective to scale)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    from prime_moe.workloads import CONFIGS
+    device = torch.device("cuda:0")
+    log = lambda *a: print(*a, file=sys.stderr, flush=True)
+    log(f"device: {torch.cuda.get_device_name(0)}; peaks used: bf16 {PEAK_TFLOPS['bf16']} / "
+        f"mxfp8 {PEAK_TFLOPS['mxfp8']} TFLOP/s dense, HBM {PEAK_HBM_GBS} GB/s")
+    if args.all:
+        for name, cfg in CONFIGS.items():
+            if name == args.config:
+                continue
+            for split in (1, 0):
+                n_steps = max(5, args.steps // 2)
+                run_config(cfg, split, n_steps, 2, device, False, log)
+                torch.cuda.empty_cache()
+    cfg = CONFIGS[args.config]
+    r = run_config(cfg, args.split, args.steps, args.warmup, device,
+                   with_cpu=(not args.no_cpu and cfg.dtype == "bf16"), log=log)
+    memory_bound = cfg.name.startswith("c5")
+    if memory_bound:
+        roofline = {"bound": "hbm", "achieved": r["bytes"] / r["ev_mean"] / 1e9, "peak": PEAK_HBM_GBS,
+                    "unit": "GB/s", "kernel": "whole op"}
+    else:
+        P = cfg.T * cfg.top_k
+        roofline = {"bound": "mfma", "achieved": 2.0 * P * cfg.K * cfg.N / r["t_up"] / 1e12,
+                    "peak": PEAK_TFLOPS[cfg.dtype], "unit": "TFLOP/s",
+                    "kernel": "moe_up_kernel (gate/up GEMM + SwiGLU)", "launch_us": r["t_up"] * 1e6}
+    roofline["frac"] = roofline["achieved"] / roofline["peak"]
+    roofline["traffic"] = None
+    line = {
+        "metric": "Fused-MoE TFLOP/s & % MFMA peak (bf16/mxfp8); decode-shape HBM GB/s",
+        "value": r["weight_gbs"] if memory_bound else r["tflops"],
+        "unit": "GB/s" if memory_bound else "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["sec"] * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": cfg.dtype, "data": "synthetic",
+        "config": {"workload": f"{cfg.name}: T={cfg.T} K={cfg.K} E={cfg.E} N={cfg.N} top_k={cfg.top_k} "
+                               f"block_m=128 split={bool(args.split)}",
+                   "flops_per_step": cfg.flops, "pct_mfma_peak": r["pct_mfma"],
+                   "weight_gbs": r["weight_gbs"], "parity_rel_clamp_1": r["parity"]},
+        "roofline": roofline,
+        "cpu_baseline": r["cpu"],
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,668 @@
+// Fused MoE forward for gfx950: gate/up grouped GEMM + SwiGLU (+ on-chip MX requantisation),
+// down GEMM with the routing-weight reduction, for bf16 and mxfp8 operands.
+//
+// Replaces the launchers and kernels of the reference's
+// prime_moe/csrc/kernels/fused_moe_bf16_kernel.cu:21-733 and fused_moe_mxfp8_kernel.cu:56-866.
+//
+// Pipelines
+//   split != 0 : zero(accum) -> up kernel (act tile -> workspace) -> down kernel (fp32 atomics
+//                into accum, one addend per routed pair) -> finalize (out = bf16(accum)).
+//   split == 0 : zero(accum) -> fused kernel: up phase leaves the 128x128 activation tile in LDS
+//                in MFMA operand layout, the down phase streams W2[e][:, h-slice] against it and
+//                adds every 128x256 partial product into accum (split-K over H/128 workgroups)
+//                -> finalize (out += bf16(accum)).
+// The top-k reduction is exact in fp32 up to summation order; `out` is rounded to bf16 once.
+#include <algorithm>
+
+#include "moe_tile.h"
+#include "pmoe_common.h"
+
+namespace pmoe {
+
+struct MoeArgs {
+    const char *x;
+    const uint8_t *x_scales;
+    const char *w1;
+    const uint8_t *w1_scales;
+    const char *w2;
+    const uint8_t *w2_scales;
+    const int32_t *sorted_ids;
+    const int32_t *expert_ids;
+    const int32_t *ntpp;
+    const float *topk_w;
+    char *act;            // (sorted_num, H) activation workspace (split pipeline)
+    uint8_t *act_scales;  // (sorted_num, H/32) e8m0, row major (mxfp8 split pipeline)
+    float *accum;         // (M, K) fp32 accumulator
+    int top_k, M, K, N, H, E, sorted_num;
+    int n_blocks;  // sorted_num / 128 (rounded up)
+    int n_wtiles;  // weight tiles along the free dimension: H/128 (up) or ceil(K/256) (down)
+};
+
+constexpr int kActPitchBf16 = 272;  // 128 bf16 + 16 B pad: 16-byte aligned rows, 2-way conflicts at most
+constexpr int kActPitchFp8 = 144;   // 128 e4m3 + 16 B pad
+
+// Logical tile id -> (row block, weight tile).  Hardware hands consecutive workgroup ids to the
+// 8 XCDs round-robin; ids are first regrouped so that one XCD runs a contiguous range of logical
+// ids, then a range is walked as [group of 4 weight tiles][row blocks][tile in group] so the 32
+// tiles resident on an XCD share x rows 4 ways and (for experts spanning several row blocks) the
+// weight slice several ways inside that XCD's L2.
+__device__ __forceinline__ bool map_tile(const MoeArgs &a, int &blk, int &wt) {
+    const int G = a.n_blocks * a.n_wtiles;
+    const int per_xcd = (int)(gridDim.x >> 3);
+    const int logical = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if (logical >= G) return false;
+    constexpr int GW = 4;
+    const int full = a.n_wtiles / GW * GW;
+    const int per_group = a.n_blocks * GW;
+    const int g = logical / per_group;
+    if (g * GW < full) {
+        const int rem = logical - g * per_group;
+        blk = rem / GW;
+        wt = g * GW + rem % GW;
+    } else {
+        const int tw = a.n_wtiles - full;
+        const int rem = logical - (full / GW) * per_group;
+        blk = rem / tw;
+        wt = full + rem % tw;
+    }
+    return true;
+}
+
+struct RowInfo {
+    int tok[kTokRows];    // token index of each sorted row, -1 for padding / dropped rows
+    float wt[kTokRows];   // routing weight of the row's pair
+    int nvalid;           // 1 + index of the last live row
+};
+
+// Fills RowInfo for row block `blk`; returns the number of 32-row fragments holding live rows.
+__device__ __forceinline__ int load_row_info(const MoeArgs &a, int blk, RowInfo &ri) {
+    const int tid = threadIdx.x;
+    if (tid == 0) ri.nvalid = 0;
+    __syncthreads();
+    if (tid < kTokRows) {
+        const int s = blk * kTokRows + tid;
+        int p = (s < a.sorted_num) ? a.sorted_ids[s] : -1;
+        int tok = -1;
+        float wt = 0.f;
+        if (p >= 0) {
+            tok = p / a.top_k;
+            if (tok < a.M) wt = a.topk_w[p];
+            else tok = -1;
+        }
+        ri.tok[tid] = tok;
+        ri.wt[tid] = wt;
+        if (tok >= 0) atomicMax(&ri.nvalid, tid + 1);
+    }
+    __syncthreads();
+    return (ri.nvalid + 31) >> 5;
+}
+
+template <int DT>
+struct ScaleRegs {
+    uint32_t tok[4];
+    uint32_t w[2];
+};
+
+// K loop of one tile: double-buffered LDS stages, prefetch of slab k+1 while slab k computes.
+template <int DT, int NTF, bool TRANSPOSED>
+__device__ __forceinline__ void tile_main_loop(f32x16 (&acc)[2][4], StageLoader &ld, char *lds,
+                                               int n_slabs, const int (&wrow)[2], int lane,
+                                               const uint8_t *const (&tok_sc)[4],
+                                               const uint8_t *const (&w_sc)[2]) {
+    uint32_t stok[4] = {0, 0, 0, 0}, sw[2] = {0, 0};
+    uint32_t ntok[4] = {0, 0, 0, 0}, nw[2] = {0, 0};
+    ld.template load<NTF>(0);
+    if constexpr (DT == DT_FP8) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if (t < NTF) stok[t] = *reinterpret_cast<const uint32_t *>(tok_sc[t]);
+#pragma unroll
+        for (int f = 0; f < 2; ++f) sw[f] = *reinterpret_cast<const uint32_t *>(w_sc[f]);
+    }
+    ld.template store_tok<NTF>(lds);
+    ld.store_w(lds);
+    __syncthreads();
+    for (int kt = 0; kt < n_slabs; ++kt) {
+        char *cur = lds + (kt & 1) * kStageBytes;
+        char *nxt = lds + ((kt + 1) & 1) * kStageBytes;
+        const bool more = kt + 1 < n_slabs;
+        if (more) {
+            ld.template load<NTF>((int64_t)(kt + 1) * kRowBytes);
+            if constexpr (DT == DT_FP8) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (t < NTF) ntok[t] = *reinterpret_cast<const uint32_t *>(tok_sc[t] + (kt + 1) * 4);
+#pragma unroll
+                for (int f = 0; f < 2; ++f)
+                    nw[f] = *reinterpret_cast<const uint32_t *>(w_sc[f] + (int64_t)(kt + 1) * 512);
+            }
+        }
+        mfma_slab<DT, NTF, TRANSPOSED>(acc, cur, cur + kTokRegion, wrow, lane, stok, sw);
+        if (more) {
+            ld.template store_tok<NTF>(nxt);
+            ld.store_w(nxt);
+            if constexpr (DT == DT_FP8) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) stok[t] = ntok[t];
+#pragma unroll
+                for (int f = 0; f < 2; ++f) sw[f] = nw[f];
+            }
+        }
+        __syncthreads();
+    }
+}
+
+__device__ __forceinline__ void zero_acc(f32x16 (&acc)[2][4]) {
+#pragma unroll
+    for (int f = 0; f < 2; ++f)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[f][t][i] = 0.f;
+}
+
+// Adds w[row] * acc into accum[token, col] for the live rows of the block.  Accumulator layout
+// (tokens on the MFMA M side): register i of lane l = row 32t + 8(i/4) + 4(l/32) + i%4,
+// column col0 + 32f + l%32, so one instruction adds two 128-byte runs.
+template <int NTF>
+__device__ __forceinline__ void scatter_add(const f32x16 (&acc)[2][4], const RowInfo &ri,
+                                            float *accum, int K, int col0, int lane) {
+    const int half = lane >> 5;
+    const int c = lane & 31;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        if (t < NTF) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int row = 32 * t + 8 * (i >> 2) + 4 * half + (i & 3);
+                const int tok = ri.tok[row];
+                const float w = ri.wt[row];
+                if (tok >= 0) {
+#pragma unroll
+                    for (int f = 0; f < 2; ++f) {
+                        const int col = col0 + 32 * f + c;
+                        if (col < K) unsafeAtomicAdd(accum + (int64_t)tok * K + col, w * acc[f][t][i]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Up kernel (and, with FUSED, the whole split==0 pipeline).
+// Tile: row block `blk` x activation columns [128*ht, 128*ht+128).  LDS weight rows 0..127 are
+// gate rows, 128..255 the matching up rows; wave v owns gate/up rows 32v..32v+31 so gate and up
+// of one activation element sit in the same lane and register.  Weight rows go on the MFMA M
+// side: a lane then holds 16 of the 32 activation columns of one MX block of its token and
+// the block maximum needs a single cross-lane exchange.
+template <int DT, bool FUSED, int NTF>
+__device__ __forceinline__ void up_tile(const MoeArgs &a, int blk, int ht, int e, RowInfo &ri,
+                                        char *lds, char *act_lds, uint32_t *act_sc_lds) {
+    constexpr int ES = DT == DT_BF16 ? 2 : 1;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, half = lane >> 5;
+    const int K = a.K, H = a.H, N = a.N;
+    const int h0 = ht * 128;
+
+    StageLoader ld;
+    const int lrow = tid >> 3, chunk = tid & 7;
+    ld.lds_off = lrow * kRowBytes + ((chunk ^ swz(lrow)) << 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int tok = ri.tok[lrow + 32 * i];
+        if (tok < 0) tok = 0;
+        ld.tok_ptr[i] = a.x + (int64_t)tok * K * ES + chunk * 16;
+    }
+    ld.w_ptr[0] = a.w1 + ((int64_t)e * N + h0 + lrow) * K * ES + chunk * 16;
+    ld.w_ptr[1] = ld.w_ptr[0] + (int64_t)H * K * ES;
+    ld.w_pitch32 = (int64_t)32 * K * ES;
+
+    const int wrow[2] = {32 * wave, 128 + 32 * wave};
+    const uint8_t *tok_sc[4] = {nullptr, nullptr, nullptr, nullptr};
+    const uint8_t *w_sc[2] = {nullptr, nullptr};
+    if constexpr (DT == DT_FP8) {
+        const int kb = K >> 5;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            int tok = ri.tok[32 * t + r];
+            if (tok < 0) tok = 0;
+            tok_sc[t] = a.x_scales + (int64_t)tok * kb;
+        }
+        const uint8_t *eb = a.w1_scales + (int64_t)e * N * kb;
+        w_sc[0] = eb + blocked_scale_off(h0 + 32 * wave + r, 0, K >> 7);
+        w_sc[1] = eb + blocked_scale_off(H + h0 + 32 * wave + r, 0, K >> 7);
+    }
+
+    f32x16 acc[2][4];
+    zero_acc(acc);
+    tile_main_loop<DT, NTF, true>(acc, ld, lds, (K * ES) / kRowBytes, wrow, lane, tok_sc, w_sc);
+
+    // ---- epilogue: SwiGLU in registers; the 2H-wide gate/up tensor never leaves the chip ----
+    // (the main loop ended with a barrier, so the stage buffers may be overwritten)
+    char *tile = FUSED ? act_lds : lds;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        if (t < NTF) {
+            float v[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) v[i] = swiglu(acc[0][t][i], acc[1][t][i]);
+            const int row = 32 * t + r;
+            if constexpr (DT == DT_BF16) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int hl = 32 * wave + 8 * g + 4 * half;  // tile-local activation column
+                    uint2 pk;
+                    pk.x = f32_to_bf16_bits(v[4 * g]) | (f32_to_bf16_bits(v[4 * g + 1]) << 16);
+                    pk.y = f32_to_bf16_bits(v[4 * g + 2]) | (f32_to_bf16_bits(v[4 * g + 3]) << 16);
+                    char *dst;
+                    if constexpr (FUSED) {
+                        const int byte = (hl & 63) * 2;
+                        dst = tile + (hl >> 6) * kTokRegion + row * kRowBytes +
+                              (((byte >> 4) ^ swz(row)) << 4) + (byte & 15);
+                    } else {
+                        dst = tile + row * kActPitchBf16 + hl * 2;
+                    }
+                    *reinterpret_cast<uint2 *>(dst) = pk;
+                }
+            } else {
+                float amax = 0.f;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(v[i]));
+                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+                uint32_t e8;
+                float inv;
+                mx_block_scale(amax, e8, inv);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int hl = 32 * wave + 8 * g + 4 * half;
+                    const uint32_t q = pack4_e4m3(v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3], inv);
+                    char *dst;
+                    if constexpr (FUSED)
+                        dst = tile + row * kRowBytes + (((hl >> 4) ^ swz(row)) << 4) + (hl & 15);
+                    else
+                        dst = tile + row * kActPitchFp8 + hl;
+                    *reinterpret_cast<uint32_t *>(dst) = q;
+                }
+                if (half == 0) reinterpret_cast<uint8_t *>(act_sc_lds)[row * 4 + wave] = (uint8_t)e8;
+            }
+        }
+    }
+    __syncthreads();
+    if constexpr (!FUSED) {
+        // coalesced copy of the live rows of the tile to the activation workspace
+        const int64_t row0 = (int64_t)blk * kTokRows;
+        if constexpr (DT == DT_BF16) {
+            const int c = tid & 15;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int row = (tid >> 4) + 16 * i;
+                if (row < 32 * NTF) {
+                    uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchBf16 + c * 16);
+                    *reinterpret_cast<uint4 *>(a.act + ((row0 + row) * H + h0) * 2 + c * 16) = v;
+                }
+            }
+        } else {
+            const int c = tid & 7;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = (tid >> 3) + 32 * i;
+                if (i < NTF) {
+                    uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchFp8 + c * 16);
+                    *reinterpret_cast<uint4 *>(a.act + (row0 + row) * H + h0 + c * 16) = v;
+                }
+            }
+            if (tid < 32 * NTF)
+                *reinterpret_cast<uint32_t *>(a.act_scales + (row0 + tid) * (H >> 5) + ht * 4) = act_sc_lds[tid];
+        }
+    }
+}
+
+// Down phase of the split==0 pipeline: the activation tile (128 rows x 128 columns of H) stays in
+// LDS as the token operand; W2[e][256-row chunk][h-slice] streams through the weight region.
+template <int DT, int NTF>
+__device__ __forceinline__ void fused_down_phase(const MoeArgs &a, int ht, int e, RowInfo &ri,
+                                                 char *lds, const char *act_lds,
+                                                 const uint32_t *act_sc_lds) {
+    constexpr int ES = DT == DT_BF16 ? 2 : 1;
+    constexpr int NS = DT == DT_BF16 ? 2 : 1;  // 128-byte slabs across the 128-column h-slice
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31;
+    const int K = a.K, H = a.H;
+    const int n_chunks = (K + kWRows - 1) / kWRows;
+    const int n_steps = n_chunks * NS;
+
+    StageLoader ld;
+    const int lrow = tid >> 3, chunk = tid & 7;
+    ld.lds_off = lrow * kRowBytes + ((chunk ^ swz(lrow)) << 4);
+    ld.w_pitch32 = (int64_t)32 * H * ES;
+    const char *w2e = a.w2 + (int64_t)e * K * H * ES + (int64_t)ht * 128 * ES + chunk * 16;
+    auto set_chunk = [&](int kc) {
+        const int k0 = kc * kWRows;
+        ld.w_ptr[0] = w2e + (int64_t)(k0 + lrow) * H * ES;
+        ld.w_ptr[1] = (k0 + 128 < K) ? ld.w_ptr[0] + (int64_t)128 * H * ES : ld.w_ptr[0];
+    };
+    const int wrow[2] = {64 * wave, 64 * wave + 32};
+    uint32_t stok[4] = {0, 0, 0, 0}, sw[2] = {0, 0};
+    const uint8_t *w2s = nullptr;
+    if constexpr (DT == DT_FP8) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if (t < NTF) stok[t] = act_sc_lds[32 * t + r];
+        w2s = a.w2_scales + (int64_t)e * K * (H >> 5);
+    }
+    auto load_wscales = [&](int kc) {
+        if constexpr (DT == DT_FP8) {
+#pragma unroll
+            for (int f = 0; f < 2; ++f) {
+                int row = kc * kWRows + 64 * wave + 32 * f + r;
+                if (row >= K) row = K - 1;
+                sw[f] = *reinterpret_cast<const uint32_t *>(w2s + blocked_scale_off(row, ht, H >> 7));
+            }
+        }
+    };
+
+    f32x16 acc[2][4];
+    set_chunk(0);
+    ld.load_w(0);
+    ld.store_w(lds);
+    __syncthreads();
+    for (int s = 0; s < n_steps; ++s) {
+        const int kc = s / NS, sl = s - kc * NS;
+        char *cur = lds + (s & 1) * kStageBytes;
+        char *nxt = lds + ((s + 1) & 1) * kStageBytes;
+        const bool more = s + 1 < n_steps;
+        if (more) {
+            const int nkc = (s + 1) / NS, nsl = (s + 1) - nkc * NS;
+            if (nsl == 0) set_chunk(nkc);
+            ld.load_w((int64_t)nsl * kRowBytes);
+        }
+        if (sl == 0) {
+            zero_acc(acc);
+            load_wscales(kc);
+        }
+        mfma_slab<DT, NTF, false>(acc, act_lds + sl * kTokRegion, cur + kTokRegion, wrow, lane, stok, sw);
+        if (sl == NS - 1) scatter_add<NTF>(acc, ri, a.accum, K, kc * kWRows + 64 * wave, lane);
+        if (more) ld.store_w(nxt);
+        __syncthreads();
+    }
+}
+
+template <int DT, bool FUSED>
+__global__ __launch_bounds__(kThreads) void moe_up_kernel(MoeArgs a) {
+    __shared__ __attribute__((aligned(1024))) char lds[kNumStages * kStageBytes];
+    __shared__ __attribute__((aligned(1024))) char act_lds[FUSED ? (DT == DT_BF16 ? 2 : 1) * kTokRegion : 16];
+    __shared__ uint32_t act_sc_lds[kTokRows];
+    __shared__ RowInfo ri;
+    int blk, ht;
+    if (!map_tile(a, blk, ht)) return;
+    if (blk * kTokRows >= a.ntpp[0]) return;
+    const int ntf = load_row_info(a, blk, ri);
+    if (ntf == 0) return;
+    const int e = a.expert_ids[blk];
+    if (e < 0 || e >= a.E) return;
+    if (ntf == 1) {
+        up_tile<DT, FUSED, 1>(a, blk, ht, e, ri, lds, act_lds, act_sc_lds);
+        if constexpr (FUSED) fused_down_phase<DT, 1>(a, ht, e, ri, lds, act_lds, act_sc_lds);
+    } else if (ntf == 2) {
+        up_tile<DT, FUSED, 2>(a, blk, ht, e, ri, lds, act_lds, act_sc_lds);
+        if constexpr (FUSED) fused_down_phase<DT, 2>(a, ht, e, ri, lds, act_lds, act_sc_lds);
+    } else {
+        up_tile<DT, FUSED, 4>(a, blk, ht, e, ri, lds, act_lds, act_sc_lds);
+        if constexpr (FUSED) fused_down_phase<DT, 4>(a, ht, e, ri, lds, act_lds, act_sc_lds);
+    }
+}
+
+// Down kernel of the split pipeline: y[128 rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
+// full reduction over H inside the workgroup (no split-K), then w[row] * y added to accum[token].
+template <int DT, int NTF>
+__device__ __forceinline__ void down_tile(const MoeArgs &a, int blk, int kt, int e, RowInfo &ri, char *lds) {
+    constexpr int ES = DT == DT_BF16 ? 2 : 1;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31;
+    const int K = a.K, H = a.H;
+    const int k0 = kt * kWRows;
+    const int64_t row0 = (int64_t)blk * kTokRows;
+
+    StageLoader ld;
+    const int lrow = tid >> 3, chunk = tid & 7;
+    ld.lds_off = lrow * kRowBytes + ((chunk ^ swz(lrow)) << 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        ld.tok_ptr[i] = a.act + (row0 + lrow + 32 * i) * H * ES + chunk * 16;
+    ld.w_ptr[0] = a.w2 + ((int64_t)e * K + k0 + lrow) * H * ES + chunk * 16;
+    ld.w_ptr[1] = (k0 + 128 < K) ? ld.w_ptr[0] + (int64_t)128 * H * ES : ld.w_ptr[0];
+    ld.w_pitch32 = (int64_t)32 * H * ES;
+
+    const int wrow[2] = {64 * wave, 64 * wave + 32};
+    const uint8_t *tok_sc[4] = {nullptr, nullptr, nullptr, nullptr};
+    const uint8_t *w_sc[2] = {nullptr, nullptr};
+    if constexpr (DT == DT_FP8) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) tok_sc[t] = a.act_scales + (row0 + 32 * t + r) * (H >> 5);
+        const uint8_t *eb = a.w2_scales + (int64_t)e * K * (H >> 5);
+#pragma unroll
+        for (int f = 0; f < 2; ++f) {
+            int row = k0 + 64 * wave + 32 * f + r;
+            if (row >= K) row = K - 1;
+            w_sc[f] = eb + blocked_scale_off(row, 0, H >> 7);
+        }
+    }
+    f32x16 acc[2][4];
+    zero_acc(acc);
+    tile_main_loop<DT, NTF, false>(acc, ld, lds, (H * ES) / kRowBytes, wrow, lane, tok_sc, w_sc);
+    scatter_add<NTF>(acc, ri, a.accum, K, k0 + 64 * wave, lane);
+}
+
+template <int DT>
+__global__ __launch_bounds__(kThreads) void moe_down_kernel(MoeArgs a) {
+    __shared__ __attribute__((aligned(1024))) char lds[kNumStages * kStageBytes];
+    __shared__ RowInfo ri;
+    int blk, kt;
+    if (!map_tile(a, blk, kt)) return;
+    if (blk * kTokRows >= a.ntpp[0]) return;
+    const int ntf = load_row_info(a, blk, ri);
+    if (ntf == 0) return;
+    const int e = a.expert_ids[blk];
+    if (e < 0 || e >= a.E) return;
+    if (ntf == 1) down_tile<DT, 1>(a, blk, kt, e, ri, lds);
+    else if (ntf == 2) down_tile<DT, 2>(a, blk, kt, e, ri, lds);
+    else down_tile<DT, 4>(a, blk, kt, e, ri, lds);
+}
+
+__global__ __launch_bounds__(256) void zero_f32_kernel(float4 *p, int64_t n4) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride)
+        p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+// out = bf16(accum)  (ACCUMULATE: out = bf16(float(out) + accum)); 8 elements per thread step.
+template <bool ACCUMULATE>
+__global__ __launch_bounds__(256) void finalize_kernel(const float4 *acc, uint4 *out, int64_t n8) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += stride) {
+        float4 lo = acc[2 * i], hi = acc[2 * i + 1];
+        float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        uint32_t o[4] = {0, 0, 0, 0};
+        if constexpr (ACCUMULATE) {
+            uint4 prev = out[i];
+            o[0] = prev.x; o[1] = prev.y; o[2] = prev.z; o[3] = prev.w;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[2 * j] += bf16_bits_to_f32(o[j] & 0xffffu);
+                v[2 * j + 1] += bf16_bits_to_f32(o[j] >> 16);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = f32_to_bf16_bits(v[2 * j]) | (f32_to_bf16_bits(v[2 * j + 1]) << 16);
+        out[i] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
+// ------------------------------------------------------------------------------------------ host
+
+struct WorkspaceLayout {
+    size_t accum_off, act_off, act_scales_off, total;
+};
+
+static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_num, int split) {
+    WorkspaceLayout l{};
+    const size_t H = (size_t)N / 2;
+    const size_t rows = align_up((size_t)sorted_num, kTokRows);
+    size_t off = 0;
+    l.accum_off = off;
+    off = align_up(off + (size_t)M * K * sizeof(float), 256);
+    l.act_off = off;
+    l.act_scales_off = off;
+    if (split) {
+        off = align_up(off + rows * H * (dt == DT_BF16 ? 2 : 1), 256);
+        l.act_scales_off = off;
+        if (dt == DT_FP8) off = align_up(off + rows * (H / 32), 256);
+    }
+    l.total = off;
+    return l;
+}
+
+static int grid_for(int n_tiles) { return (n_tiles + 7) / 8 * 8; }
+
+// Which phases of the pipeline the fused entry points enqueue (all by default); see
+// pmoe_set_phase_mask in the header.
+static thread_local int g_phase_mask = PMOE_PHASE_ALL;
+
+template <int DT>
+static int launch_pipeline(MoeArgs a, void *out, int split, hipStream_t s) {
+    const int64_t n_out = (int64_t)a.M * a.K;  // K % 128 == 0, so n_out % 8 == 0
+    const int mask = g_phase_mask;
+    if (mask & PMOE_PHASE_ZERO) {
+        const int64_t n4 = n_out / 4;
+        const int blocks = (int)std::min<int64_t>((n4 + 255) / 256, 2048);
+        hipLaunchKernelGGL(zero_f32_kernel, dim3(blocks), dim3(256), 0, s, reinterpret_cast<float4 *>(a.accum), n4);
+    }
+    a.n_blocks = (a.sorted_num + kTokRows - 1) / kTokRows;
+    a.n_wtiles = a.H / 128;
+    if (a.n_blocks > 0) {
+        const int grid = grid_for(a.n_blocks * a.n_wtiles);
+        if (split) {
+            if (mask & PMOE_PHASE_UP)
+                hipLaunchKernelGGL((moe_up_kernel<DT, false>), dim3(grid), dim3(kThreads), 0, s, a);
+            MoeArgs d = a;
+            d.n_wtiles = (a.K + kWRows - 1) / kWRows;
+            if (mask & PMOE_PHASE_DOWN)
+                hipLaunchKernelGGL((moe_down_kernel<DT>), dim3(grid_for(d.n_blocks * d.n_wtiles)), dim3(kThreads), 0, s, d);
+        } else if (mask & PMOE_PHASE_UP) {
+            hipLaunchKernelGGL((moe_up_kernel<DT, true>), dim3(grid), dim3(kThreads), 0, s, a);
+        }
+    }
+    if (mask & PMOE_PHASE_FINALIZE) {
+        const int64_t n8 = n_out / 8;
+        const int blocks = (int)std::min<int64_t>((n8 + 255) / 256, 2048);
+        if (split)
+            hipLaunchKernelGGL(finalize_kernel<false>, dim3(blocks), dim3(256), 0, s,
+                               reinterpret_cast<const float4 *>(a.accum), reinterpret_cast<uint4 *>(out), n8);
+        else
+            hipLaunchKernelGGL(finalize_kernel<true>, dim3(blocks), dim3(256), 0, s,
+                               reinterpret_cast<const float4 *>(a.accum), reinterpret_cast<uint4 *>(out), n8);
+    }
+    return check_launch("fused_moe launch");
+}
+
+}  // namespace pmoe
+
+using namespace pmoe;
+
+extern "C" void pmoe_set_phase_mask(int mask) { g_phase_mask = mask; }
+
+extern "C" size_t pmoe_fused_moe_bf16_workspace_bytes(int M, int K, int N, int num_experts,
+                                                      int sorted_num, int split) {
+    (void)num_experts;
+    if (M <= 0 || K <= 0 || N <= 0 || sorted_num < 0) return 0;
+    return workspace_layout(DT_BF16, M, K, N, sorted_num, split).total;
+}
+
+extern "C" size_t pmoe_fused_moe_mxfp8_workspace_bytes(int M, int K, int N, int num_experts,
+                                                       int sorted_num, int split) {
+    (void)num_experts;
+    if (M <= 0 || K <= 0 || N <= 0 || sorted_num < 0) return 0;
+    return workspace_layout(DT_FP8, M, K, N, sorted_num, split).total;
+}
+
+static int check_tuning(const char *op, int block_m, int block_n, int warp_n, int stages,
+                        int max_stages) {
+    PMOE_REQUIRE((block_n == 64 && warp_n == 4) || (block_n == 32 && warp_n == 8),
+                 "%s: (block_n, warp_n) must be (64, 4) or (32, 8), got (%d, %d)", op, block_n, warp_n);
+    PMOE_REQUIRE(stages > 0 && stages <= max_stages, "%s supports stages in 1..%d, got %d", op, max_stages, stages);
+    PMOE_REQUIRE(block_m == 128, "%s requires block_m=128, got %d", op, block_m);
+    return PMOE_OK;
+}
+
+extern "C" int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2, void *out,
+                                   const int32_t *sorted_token_ids, const int32_t *expert_idxs,
+                                   const int32_t *num_tokens_post_padded, const float *topk_weights,
+                                   int top_k, int M, int K, int N, int num_experts, int sorted_num,
+                                   int block_m, int block_n, int warp_n, int stages, int bpc, int cpc,
+                                   int split, void *workspace, size_t workspace_bytes, void *stream) {
+    PMOE_REQUIRE(M > 0, "fused_moe_bf16: x has no rows");
+    PMOE_REQUIRE(K > 0 && (K & 127) == 0, "K dimension must be a multiple of 128");
+    PMOE_REQUIRE(N > 0 && (N & 255) == 0, "fused_moe_bf16: N must be a multiple of 256, got %d", N);
+    if (int rc = check_tuning("fused_moe_bf16", block_m, block_n, warp_n, stages, 5)) return rc;
+    PMOE_REQUIRE(bpc == 1 && cpc == 1, "bpc=cpc=1 is the only supported configuration");
+    PMOE_REQUIRE(!split || stages <= 4, "split=True requires stages<=4, got stages=%d", stages);
+    PMOE_REQUIRE(top_k > 0 && num_experts > 0 && sorted_num >= 0, "fused_moe_bf16: bad top_k / num_experts / sorted_num");
+    PMOE_REQUIRE(x && w && w2 && out && sorted_token_ids && expert_idxs && num_tokens_post_padded && topk_weights,
+                 "fused_moe_bf16: null pointer");
+    const WorkspaceLayout l = workspace_layout(DT_BF16, M, K, N, sorted_num, split);
+    PMOE_REQUIRE(workspace && workspace_bytes >= l.total, "fused_moe_bf16: workspace of %zu bytes needed, got %zu", l.total, workspace_bytes);
+    PMOE_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, "fused_moe_bf16: workspace must be 256-byte aligned");
+    MoeArgs a{};
+    a.x = static_cast<const char *>(x);
+    a.w1 = static_cast<const char *>(w);
+    a.w2 = static_cast<const char *>(w2);
+    a.sorted_ids = sorted_token_ids;
+    a.expert_ids = expert_idxs;
+    a.ntpp = num_tokens_post_padded;
+    a.topk_w = topk_weights;
+    char *ws = static_cast<char *>(workspace);
+    a.accum = reinterpret_cast<float *>(ws + l.accum_off);
+    a.act = ws + l.act_off;
+    a.top_k = top_k; a.M = M; a.K = K; a.N = N; a.H = N / 2; a.E = num_experts; a.sorted_num = sorted_num;
+    return launch_pipeline<DT_BF16>(a, out, split, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int pmoe_fused_moe_mxfp8(const void *x, const void *x_scales, const void *w,
+                                    const void *w_scales, const void *w2, const void *w2_scales,
+                                    void *out, const int32_t *sorted_token_ids,
+                                    const int32_t *expert_idxs, const int32_t *num_tokens_post_padded,
+                                    const float *topk_weights, int top_k, int M, int K, int N,
+                                    int num_experts, int sorted_num, int block_m, int block_n,
+                                    int warp_n, int stages, int bpc, int split, void *workspace,
+                                    size_t workspace_bytes, void *stream) {
+    PMOE_REQUIRE(M > 0, "fused_moe_mxfp8: x has no rows");
+    PMOE_REQUIRE(K > 0 && (K & 255) == 0, "K dimension must be a multiple of 256 on the mxfp8 path");
+    PMOE_REQUIRE(N > 0 && (N & 255) == 0, "N dimension must be a multiple of 256 on the mxfp8 path");
+    if (int rc = check_tuning("fused_moe_mxfp8", block_m, block_n, warp_n, stages, 4)) return rc;
+    PMOE_REQUIRE(bpc == 1, "mxfp8 supports bpc=1 only");
+    PMOE_REQUIRE(top_k > 0 && num_experts > 0 && sorted_num >= 0, "fused_moe_mxfp8: bad top_k / num_experts / sorted_num");
+    PMOE_REQUIRE(x && x_scales && w && w_scales && w2 && w2_scales && out && sorted_token_ids && expert_idxs &&
+                     num_tokens_post_padded && topk_weights,
+                 "fused_moe_mxfp8: null pointer");
+    const WorkspaceLayout l = workspace_layout(DT_FP8, M, K, N, sorted_num, split);
+    PMOE_REQUIRE(workspace && workspace_bytes >= l.total, "fused_moe_mxfp8: workspace of %zu bytes needed, got %zu", l.total, workspace_bytes);
+    PMOE_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, "fused_moe_mxfp8: workspace must be 256-byte aligned");
+    MoeArgs a{};
+    a.x = static_cast<const char *>(x);
+    a.x_scales = static_cast<const uint8_t *>(x_scales);
+    a.w1 = static_cast<const char *>(w);
+    a.w1_scales = static_cast<const uint8_t *>(w_scales);
+    a.w2 = static_cast<const char *>(w2);
+    a.w2_scales = static_cast<const uint8_t *>(w2_scales);
+    a.sorted_ids = sorted_token_ids;
+    a.expert_ids = expert_idxs;
+    a.ntpp = num_tokens_post_padded;
+    a.topk_w = topk_weights;
+    char *ws = static_cast<char *>(workspace);
+    a.accum = reinterpret_cast<float *>(ws + l.accum_off);
+    a.act = ws + l.act_off;
+    a.act_scales = reinterpret_cast<uint8_t *>(ws + l.act_scales_off);
+    a.top_k = top_k; a.M = M; a.K = K; a.N = N; a.H = N / 2; a.E = num_experts; a.sorted_num = sorted_num;
+    return launch_pipeline<DT_FP8>(a, out, split, static_cast<hipStream_t>(stream));
+}

@@ -1,0 +1,157 @@
+// moe_align for gfx950: stable counting sort of pair ids by expert, padded per expert.
+//
+// Semantics follow the reference kernel (prime_moe/csrc/kernels/fused_moe_bf16_kernel.cu:853-907)
+// except that the within-expert order is made unique (ascending pair id) instead of being
+// left to an atomic race.  One workgroup, wave64:
+//   1. each wave histograms a contiguous slice of the ids into its own LDS row,
+//   2. per expert, the per-wave counts become exclusive per-wave bases; the padded
+//      per-expert totals are prefix-summed by one wave with a shuffle scan,
+//   3. each wave walks its slice again 64 ids at a time; lanes holding the same
+//      expert find each other with one ballot per id bit, the lane's rank inside
+//      that group is a popcount of the lower lanes, and the destination is
+//      offs[e] + base[wave][e] + rank.
+// All arithmetic is int32 and the output is a pure function of the input.
+#include "pmoe_common.h"
+
+namespace {
+
+constexpr int kMaxExperts = 1024;
+
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void moe_align_kernel(
+    const int32_t *__restrict__ topk_ids, int32_t *__restrict__ sorted_token_ids,
+    int32_t *__restrict__ expert_ids, int32_t *__restrict__ num_tokens_post_padded, int n,
+    int num_experts, int block_m, int pad_to, int max_padded, int max_blocks, int id_bits) {
+    extern __shared__ int32_t smem[];
+    int32_t *offs = smem;                          // [E+1] exclusive prefix of padded counts
+    int32_t *padc = smem + (num_experts + 1);      // [E]   padded count per expert
+    int32_t *wbase = smem + (2 * num_experts + 1);  // [NW][E] per-wave counts, then running bases
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    constexpr int NT = NW * 64;
+    const int E = num_experts;
+
+    for (int i = tid; i < NW * E; i += NT) wbase[i] = 0;
+    __syncthreads();
+
+    // contiguous slice per wave, a multiple of 64 ids so groups never straddle waves
+    const int per_wave = (n + NT - 1) / NT * 64;
+    const int beg = wave * per_wave;
+    const int end = min(n, beg + per_wave);
+    int32_t *mine = wbase + wave * E;
+    for (int i = beg + lane; i < end; i += 64) {
+        int e = topk_ids[i];
+        if (e >= 0 && e < E) atomicAdd(mine + e, 1);
+    }
+    __syncthreads();
+
+    // per expert: counts of the waves -> exclusive bases; padded total of the expert
+    for (int e = tid; e < E; e += NT) {
+        int run = 0;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            int c = wbase[w * E + e];
+            wbase[w * E + e] = run;
+            run += c;
+        }
+        padc[e] = (run + pad_to - 1) / pad_to * pad_to;
+    }
+    __syncthreads();
+
+    // exclusive prefix over experts by wave 0: serial inside a lane's chunk, shuffle scan across
+    if (wave == 0) {
+        const int chunk = (E + 63) >> 6;
+        const int b = lane * chunk;
+        int local = 0;
+        for (int j = 0; j < chunk; ++j)
+            if (b + j < E) local += padc[b + j];
+        int incl = local;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            int v = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += v;
+        }
+        int run = incl - local;
+        for (int j = 0; j < chunk; ++j)
+            if (b + j < E) {
+                offs[b + j] = run;
+                run += padc[b + j];
+            }
+        if (lane == 63) offs[E] = incl;  // lane 63's inclusive sum is the grand total
+    }
+    __syncthreads();
+    const int total = offs[E];
+    if (tid == 0) num_tokens_post_padded[0] = total;
+
+    for (int i = tid; i < max_padded; i += NT) sorted_token_ids[i] = -1;
+    for (int j = tid; j < max_blocks; j += NT) {
+        const int row = j * block_m;
+        int owner = E - 1;
+        if (row < total) {
+            int lo = 0, hi = E - 1;
+            while (lo < hi) {
+                int mid = (lo + hi + 1) >> 1;
+                if (offs[mid] <= row) lo = mid;
+                else hi = mid - 1;
+            }
+            owner = lo;
+        }
+        expert_ids[j] = owner;
+    }
+    __syncthreads();  // the -1 fill is complete before any pair id lands on top of it
+
+    for (int i0 = beg; i0 < end; i0 += 64) {
+        const int i = i0 + lane;
+        int e = (i < end) ? topk_ids[i] : -1;
+        const bool valid = e >= 0 && e < E;
+        unsigned long long peers = __ballot(valid);
+        for (int b = 0; b < id_bits; ++b) {
+            const bool bit = (e >> b) & 1;
+            const unsigned long long set = __ballot(bit);
+            peers &= bit ? set : ~set;
+        }
+        if (valid) {
+            const int rank = __popcll(peers & ((1ull << lane) - 1ull));
+            const int cnt = __popcll(peers);
+            const int base = mine[e];
+            sorted_token_ids[offs[e] + base + rank] = i;
+            if (rank == cnt - 1) mine[e] = base + cnt;  // one writer per group, after all reads
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int pmoe_moe_align(const int32_t *topk_ids, int32_t *sorted_token_ids,
+                              int32_t *expert_ids, int32_t *num_tokens_post_padded, int n,
+                              int num_experts, int block_m, int pad_to, int max_padded,
+                              int max_blocks, void *stream) {
+    PMOE_REQUIRE(num_experts > 0 && block_m > 0 && pad_to > 0, "moe_align: block_m, bpc and num_experts must be positive");
+    PMOE_REQUIRE(num_experts <= kMaxExperts, "moe_align supports at most 1024 experts, got %d", num_experts);
+    PMOE_REQUIRE(n >= 0 && max_padded >= 0 && max_blocks >= 0, "moe_align: negative size");
+    PMOE_REQUIRE(pad_to % block_m == 0, "moe_align: pad_to must be a multiple of block_m");
+    {
+        const long long need = ((long long)n + (long long)num_experts * (pad_to - 1) + pad_to - 1) / pad_to * pad_to;
+        PMOE_REQUIRE(max_padded >= need, "moe_align: max_padded %d is smaller than the worst case %lld", max_padded, need);
+        PMOE_REQUIRE((long long)max_blocks * block_m <= (long long)max_padded + block_m - 1, "moe_align: max_blocks %d does not match max_padded %d", max_blocks, max_padded);
+    }
+    PMOE_REQUIRE(sorted_token_ids && expert_ids && num_tokens_post_padded && (topk_ids || n == 0), "moe_align: null pointer");
+    int id_bits = 1;
+    while ((1 << id_bits) < num_experts) ++id_bits;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (num_experts <= 512) {
+        constexpr int NW = 16;
+        size_t smem = sizeof(int32_t) * (size_t)(2 * num_experts + 1 + NW * num_experts);
+        hipLaunchKernelGGL(moe_align_kernel<NW>, dim3(1), dim3(NW * 64), smem, s, topk_ids,
+                           sorted_token_ids, expert_ids, num_tokens_post_padded, n, num_experts,
+                           block_m, pad_to, max_padded, max_blocks, id_bits);
+    } else {
+        constexpr int NW = 8;
+        size_t smem = sizeof(int32_t) * (size_t)(2 * num_experts + 1 + NW * num_experts);
+        hipLaunchKernelGGL(moe_align_kernel<NW>, dim3(1), dim3(NW * 64), smem, s, topk_ids,
+                           sorted_token_ids, expert_ids, num_tokens_post_padded, n, num_experts,
+                           block_m, pad_to, max_padded, max_blocks, id_bits);
+    }
+    return pmoe::check_launch("moe_align launch");
+}

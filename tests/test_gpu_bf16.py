@@ -1,0 +1,137 @@
+"""fused_moe_bf16 on the GPU vs the fp32 CPU oracle on identical seeded inputs.
+Gate: max |got - ref| / max(|ref|, 1) <= 2e-2."""
+import math
+
+import pytest
+import torch
+
+from helpers import BF16_GATE, oracle_schedule, reference_routing, rel_clamp
+from oracle import moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(T, K, E, N, device, seed, x_std=1.0):
+    g = torch.Generator(device=device).manual_seed(seed)
+    x = (torch.randn((T, K), device=device, generator=g) * x_std).to(torch.bfloat16)
+    w1 = (torch.randn((E, N, K), device=device, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    w2 = (torch.randn((E, K, N // 2), device=device, generator=g) / math.sqrt(N // 2)).to(torch.bfloat16)
+    return g, x, w1, w2
+
+
+def _run_case(T, K, E, N, top_k, split, device, seed=0, use_op_align=True, exact=False, hot_last=True,
+              prefill_out=None):
+    import prime_moe
+    g, x, w1, w2 = _inputs(T, K, E, N, device, seed)
+    ids, wts = reference_routing(T, E, top_k, device, g, hot_last=hot_last)
+    if use_op_align:
+        sched = torch.ops.prime_moe.moe_align(ids, E, 128, 1)
+    else:
+        sched = oracle_schedule(ids, E, 128, exact=exact)
+    if prefill_out is None:
+        out = torch.zeros((T, K), dtype=torch.bfloat16, device=device) if not split else \
+            torch.full((T, K), float("nan"), dtype=torch.bfloat16, device=device)
+    else:
+        out = prefill_out.clone()
+    ret = prime_moe.fused_moe_bf16(x, w1, w2, *sched, wts, out, top_k, 128, 64, 4, 2, 1, 1, split)
+    torch.cuda.synchronize()
+    assert ret is out
+    ref = O.fused_moe_dense(x.cpu(), w1.cpu(), w2.cpu(), ids.cpu(), wts.cpu())
+    if prefill_out is not None and not split:
+        ref = ref + prefill_out.float().cpu()
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    err = rel_clamp(got, ref, 1.0)
+    assert err <= BF16_GATE, f"rel_clamp_1 {err:.4g} > {BF16_GATE}"
+    return err
+
+
+@pytest.mark.parametrize("split", [True, False])
+def test_readme_shape(split, device):
+    # T=256 K=4096 E=8 N=512 top_k=4 with top-4 of N(0,1) logits and softmax weights
+    import prime_moe
+    from prime_moe.workloads import CONFIGS, make_inputs
+    cfg = CONFIGS["c1_readme_bf16"]
+    inp = make_inputs(cfg, device, seed=1)
+    sched = torch.ops.prime_moe.moe_align(inp["topk_ids"], cfg.E, 128, 1)
+    out = torch.zeros((cfg.T, cfg.K), dtype=torch.bfloat16, device=device)
+    prime_moe.fused_moe_bf16(inp["x"], inp["w1"], inp["w2"], *sched, inp["topk_weights"], out, cfg.top_k,
+                             128, 64, 4, 2, 1, 1, split)
+    torch.cuda.synchronize()
+    ref = O.fused_moe_dense(inp["x"].cpu(), inp["w1"].cpu(), inp["w2"].cpu(), inp["topk_ids"].cpu(),
+                            inp["topk_weights"].cpu())
+    err = rel_clamp(out.float().cpu(), ref, 1.0)
+    assert err <= BF16_GATE, err
+
+
+@pytest.mark.parametrize("split", [True, False])
+@pytest.mark.parametrize("T,K,E,N", [
+    (8, 4096, 257, 256), (32, 7168, 8, 512), (128, 4096, 37, 256), (256, 7168, 37, 512),
+    (200, 1024, 8, 768), (1, 128, 1, 256), (130, 384, 3, 256),
+])
+def test_reference_sweep_shapes(T, K, E, N, split, device):
+    # the reference's own sweep grid (test/test.py:133-146), top_k = 9 with a hot last expert,
+    # plus ragged cases: K % 256 == 128, a single token, one expert
+    top_k = 9 if E > 1 else 1
+    _run_case(T, K, E, N, top_k, split, device, seed=T + E)
+
+
+@pytest.mark.parametrize("split", [True, False])
+def test_exact_size_schedule_from_python_restatement(split, device):
+    _run_case(64, 1024, 8, 512, 4, split, device, use_op_align=False, exact=True)
+    _run_case(64, 1024, 8, 512, 4, split, device, use_op_align=False, exact=False)
+
+
+def test_split_overwrites_and_fused_accumulates(device):
+    T, K = 96, 512
+    pre = torch.randn((T, K), device=device).to(torch.bfloat16)
+    _run_case(T, K, 4, 256, 2, True, device, prefill_out=pre, hot_last=False)   # overwritten
+    _run_case(T, K, 4, 256, 2, False, device, prefill_out=pre, hot_last=False)  # added to
+
+
+def test_tokens_beyond_m_are_dropped(device):
+    import prime_moe
+    T, K, E, N, top_k = 64, 512, 4, 256, 2
+    g, x, w1, w2 = _inputs(T, K, E, N, device, 3)
+    ids, wts = reference_routing(T, E, top_k, device, g, hot_last=False)
+    sched = torch.ops.prime_moe.moe_align(ids, E, 128, 1)
+    keep = 40  # x with fewer rows than the schedule refers to: rows of tokens >= keep are skipped
+    out = torch.zeros((keep, K), dtype=torch.bfloat16, device=device)
+    prime_moe.fused_moe_bf16(x[:keep].contiguous(), w1, w2, *sched, wts, out, top_k, 128, 32, 8, 1, 1, 1, True)
+    torch.cuda.synchronize()
+    ref = O.fused_moe_dense(x.cpu(), w1.cpu(), w2.cpu(), ids.cpu(), wts.cpu())[:keep]
+    assert rel_clamp(out.float().cpu(), ref, 1.0) <= BF16_GATE
+
+
+def test_validation_errors(device):
+    import prime_moe
+    T, K, E, N, top_k = 16, 256, 2, 256, 2
+    g, x, w1, w2 = _inputs(T, K, E, N, device, 0)
+    ids, wts = reference_routing(T, E, top_k, device, g, hot_last=False)
+    sched = torch.ops.prime_moe.moe_align(ids, E, 128, 1)
+    out = torch.zeros((T, K), dtype=torch.bfloat16, device=device)
+    ok = dict(top_k=top_k, block_m=128, block_n=64, warp_n=4, stages=2, bpc=1, cpc=1, split=True)
+
+    def call(**kw):
+        a = dict(ok)
+        a.update(kw)
+        prime_moe.fused_moe_bf16(kw.pop("x", x), w1, w2, *sched, kw.pop("wts", wts), kw.pop("out", out),
+                                 a["top_k"], a["block_m"], a["block_n"], a["warp_n"], a["stages"], a["bpc"],
+                                 a["cpc"], a["split"])
+
+    call()
+    for bad in (dict(block_m=64), dict(block_n=64, warp_n=8), dict(stages=0), dict(stages=6),
+                dict(stages=5, split=True), dict(bpc=2), dict(cpc=2)):
+        with pytest.raises(RuntimeError):
+            call(**bad)
+    call(stages=5, split=False)
+    with pytest.raises(RuntimeError):
+        call(x=x.float())
+    with pytest.raises(RuntimeError):
+        call(out=out.float())
+    with pytest.raises(RuntimeError):
+        call(wts=wts.double())
+    with pytest.raises(RuntimeError):
+        call(x=x.t().contiguous().t())
+    with pytest.raises(RuntimeError):
+        call(x=x[:, :192].contiguous())

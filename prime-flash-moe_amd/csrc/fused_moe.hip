@@ -13,6 +13,7 @@
 //                -> finalize (out += bf16(accum)).
 // The top-k reduction is exact in fp32 up to summation order; `out` is rounded to bf16 once.
 #include <algorithm>
+#include <type_traits>
 
 #include "moe_tile.h"
 #include "pmoe_common.h"
@@ -33,6 +34,8 @@ struct MoeArgs {
     char *act;            // (sorted_num, H) activation workspace (split pipeline)
     uint8_t *act_scales;  // (sorted_num, H/32) e8m0, row major (mxfp8 split pipeline)
     float *accum;         // (M, K) fp32 accumulator
+    const int2 *tiles;    // row tiles built by the prologue: (first block, number of blocks 1..2)
+    const int *n_tiles;   // number of row tiles
     int top_k, M, K, N, H, E, sorted_num;
     int n_blocks;  // sorted_num / 128 (rounded up)
     int n_wtiles;  // weight tiles along the free dimension: H/128 (up) or ceil(K/256) (down)
@@ -41,107 +44,133 @@ struct MoeArgs {
 constexpr int kActPitchBf16 = 272;  // 128 bf16 + 16 B pad: 16-byte aligned rows, 2-way conflicts at most
 constexpr int kActPitchFp8 = 144;   // 128 e4m3 + 16 B pad
 
-// Logical tile id -> (row block, weight tile).  Hardware hands consecutive workgroup ids to the
-// 8 XCDs round-robin; ids are first regrouped so that one XCD runs a contiguous range of logical
-// ids, then a range is walked as [group of 4 weight tiles][row blocks][tile in group] so the 32
-// tiles resident on an XCD share x rows 4 ways and (for experts spanning several row blocks) the
-// weight slice several ways inside that XCD's L2.
-__device__ __forceinline__ bool map_tile(const MoeArgs &a, int &blk, int &wt) {
-    const int G = a.n_blocks * a.n_wtiles;
-    const int per_xcd = (int)(gridDim.x >> 3);
-    const int logical = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+// Workgroup id -> (row tile, weight tile), using the live tile count read on the device.
+// Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; ids are regrouped so that
+// one XCD runs a contiguous range of logical ids, and a range is walked as
+// [group of GW weight tiles][row tiles][weight tile in group]: the ~32 tiles resident on an XCD
+// then share their token rows GW ways and, for experts spanning several row tiles, their weight
+// slice several ways inside that XCD's L2.
+template <int NG>
+__device__ __forceinline__ bool resolve_tile(const MoeArgs &a, int &first, int &nb, int &wt) {
+    int n_row_tiles;
+    if constexpr (NG == 2) n_row_tiles = min(a.n_tiles[0], a.n_blocks);
+    else n_row_tiles = min((a.ntpp[0] + kBlockRows - 1) / kBlockRows, a.n_blocks);
+    const int G = n_row_tiles * a.n_wtiles;
+    const int per_xcd = (G + 7) >> 3;
+    const int idx = (int)(blockIdx.x >> 3);
+    if (idx >= per_xcd) return false;
+    const int logical = (int)(blockIdx.x & 7) * per_xcd + idx;
     if (logical >= G) return false;
-    constexpr int GW = 4;
+    constexpr int GW = 8;
     const int full = a.n_wtiles / GW * GW;
-    const int per_group = a.n_blocks * GW;
+    const int per_group = n_row_tiles * GW;
     const int g = logical / per_group;
+    int rt;
     if (g * GW < full) {
         const int rem = logical - g * per_group;
-        blk = rem / GW;
+        rt = rem / GW;
         wt = g * GW + rem % GW;
     } else {
         const int tw = a.n_wtiles - full;
         const int rem = logical - (full / GW) * per_group;
-        blk = rem / tw;
+        rt = rem / tw;
         wt = full + rem % tw;
+    }
+    if constexpr (NG == 2) {
+        const int2 t = a.tiles[rt];
+        first = t.x;
+        nb = t.y;
+    } else {
+        first = rt;
+        nb = 1;
     }
     return true;
 }
 
+template <int NG>
 struct RowInfo {
-    int tok[kTokRows];    // token index of each sorted row, -1 for padding / dropped rows
-    float wt[kTokRows];   // routing weight of the row's pair
-    int nvalid;           // 1 + index of the last live row
+    int tok[kBlockRows * NG];   // token index of each sorted row, -1 for padding / dropped rows
+    float wt[kBlockRows * NG];  // routing weight of the row's pair
+    int nvalid[NG];             // per group: 1 + index of the last live row
 };
 
-// Fills RowInfo for row block `blk`; returns the number of 32-row fragments holding live rows.
-__device__ __forceinline__ int load_row_info(const MoeArgs &a, int blk, RowInfo &ri) {
+// Fills RowInfo for the `nb` blocks starting at `first`; returns the largest number of 32-row
+// fragments holding live rows in any group.
+template <int NG>
+__device__ __forceinline__ int load_row_info(const MoeArgs &a, int first, int nb, RowInfo<NG> &ri) {
     const int tid = threadIdx.x;
-    if (tid == 0) ri.nvalid = 0;
+    if (tid < NG) ri.nvalid[tid] = 0;
     __syncthreads();
-    if (tid < kTokRows) {
-        const int s = blk * kTokRows + tid;
-        int p = (s < a.sorted_num) ? a.sorted_ids[s] : -1;
+    if (tid < kBlockRows * NG) {
+        const int g = tid >> 7;
         int tok = -1;
         float wt = 0.f;
-        if (p >= 0) {
-            tok = p / a.top_k;
-            if (tok < a.M) wt = a.topk_w[p];
-            else tok = -1;
+        if (g < nb) {
+            const int s = first * kBlockRows + tid;
+            const int p = (s < a.sorted_num) ? a.sorted_ids[s] : -1;
+            if (p >= 0) {
+                tok = p / a.top_k;
+                if (tok < a.M) wt = a.topk_w[p];
+                else tok = -1;
+            }
         }
         ri.tok[tid] = tok;
         ri.wt[tid] = wt;
-        if (tok >= 0) atomicMax(&ri.nvalid, tid + 1);
+        if (tok >= 0) atomicMax(&ri.nvalid[g], (tid & 127) + 1);
     }
     __syncthreads();
-    return (ri.nvalid + 31) >> 5;
+    int m = 0;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) m = max(m, (ri.nvalid[g] + 31) >> 5);
+    return m;
 }
 
-template <int DT>
-struct ScaleRegs {
-    uint32_t tok[4];
-    uint32_t w[2];
-};
-
 // K loop of one tile: double-buffered LDS stages, prefetch of slab k+1 while slab k computes.
-template <int DT, int NTF, bool TRANSPOSED>
-__device__ __forceinline__ void tile_main_loop(f32x16 (&acc)[2][4], StageLoader &ld, char *lds,
-                                               int n_slabs, const int (&wrow)[2], int lane,
-                                               const uint8_t *const (&tok_sc)[4],
-                                               const uint8_t *const (&w_sc)[2]) {
+// COMPUTE = false is the loop of the waves of a group without live rows: they only take part in
+// the copies and barriers (same barrier count, no matrix work, no accumulator traffic).
+template <int DT, int NG, int NTF, bool TRANSPOSED, bool COMPUTE>
+__device__ __forceinline__ void tile_main_loop(f32x16 (&acc)[2][4], StageLoader<NG> &ld, char *lds,
+                                               int n_slabs, const int (&wrow)[2], int lane, int grp,
+                                               const uint8_t *tok_sc_base,
+                                               const uint32_t (&tok_sc)[4], const uint8_t *w_sc_base,
+                                               const uint32_t (&w_sc)[2]) {
+    using G = Geo<NG>;
     uint32_t stok[4] = {0, 0, 0, 0}, sw[2] = {0, 0};
     uint32_t ntok[4] = {0, 0, 0, 0}, nw[2] = {0, 0};
-    ld.template load<NTF>(0);
-    if constexpr (DT == DT_FP8) {
+    ld.load_tok(0);
+    ld.load_w(0);
+    if constexpr (DT == DT_FP8 && COMPUTE) {
 #pragma unroll
         for (int t = 0; t < 4; ++t)
-            if (t < NTF) stok[t] = *reinterpret_cast<const uint32_t *>(tok_sc[t]);
+            if (t < NTF) stok[t] = *reinterpret_cast<const uint32_t *>(tok_sc_base + tok_sc[t]);
 #pragma unroll
-        for (int f = 0; f < 2; ++f) sw[f] = *reinterpret_cast<const uint32_t *>(w_sc[f]);
+        for (int f = 0; f < 2; ++f) sw[f] = *reinterpret_cast<const uint32_t *>(w_sc_base + w_sc[f]);
     }
-    ld.template store_tok<NTF>(lds);
+    ld.store_tok(lds);
     ld.store_w(lds);
     __syncthreads();
     for (int kt = 0; kt < n_slabs; ++kt) {
-        char *cur = lds + (kt & 1) * kStageBytes;
-        char *nxt = lds + ((kt + 1) & 1) * kStageBytes;
+        char *cur = lds + (kt & 1) * G::kStageBytes;
+        char *nxt = lds + ((kt + 1) & 1) * G::kStageBytes;
         const bool more = kt + 1 < n_slabs;
         if (more) {
-            ld.template load<NTF>((int64_t)(kt + 1) * kRowBytes);
-            if constexpr (DT == DT_FP8) {
+            ld.load_tok((uint32_t)(kt + 1) * kRowBytes);
+            ld.load_w((uint32_t)(kt + 1) * kRowBytes);
+            if constexpr (DT == DT_FP8 && COMPUTE) {
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
-                    if (t < NTF) ntok[t] = *reinterpret_cast<const uint32_t *>(tok_sc[t] + (kt + 1) * 4);
+                    if (t < NTF) ntok[t] = *reinterpret_cast<const uint32_t *>(tok_sc_base + (tok_sc[t] + (uint32_t)(kt + 1) * 4));
 #pragma unroll
                 for (int f = 0; f < 2; ++f)
-                    nw[f] = *reinterpret_cast<const uint32_t *>(w_sc[f] + (int64_t)(kt + 1) * 512);
+                    nw[f] = *reinterpret_cast<const uint32_t *>(w_sc_base + (w_sc[f] + (uint32_t)(kt + 1) * 512));
             }
         }
-        mfma_slab<DT, NTF, TRANSPOSED>(acc, cur, cur + kTokRegion, wrow, lane, stok, sw);
+        if constexpr (COMPUTE)
+            mfma_slab<DT, NTF, TRANSPOSED, NG == 1>(acc, cur + grp * kGroupRegion, cur + G::kTokRegion, wrow, lane, stok, sw);
         if (more) {
-            ld.template store_tok<NTF>(nxt);
+            ld.store_tok(nxt);
             ld.store_w(nxt);
-            if constexpr (DT == DT_FP8) {
+            if constexpr (DT == DT_FP8 && COMPUTE) {
 #pragma unroll
                 for (int t = 0; t < 4; ++t) stok[t] = ntok[t];
 #pragma unroll
@@ -150,6 +179,86 @@ __device__ __forceinline__ void tile_main_loop(f32x16 (&acc)[2][4], StageLoader 
         }
         __syncthreads();
     }
+}
+
+// K loop of the two-group kernels: the next slab is copied global -> LDS by the DMA path while the
+// current one is consumed, one barrier per slab.  For bf16 the MFMAs are software-pipelined across
+// that barrier: the last K sub-step of a slab is held back and issued after the barrier, behind the
+// first fragment reads of the next slab, so the matrix pipe has work while LDS latency elapses.
+template <int DT, int NG, int NTF, bool TRANSPOSED, bool COMPUTE>
+__device__ __forceinline__ void tile_main_loop_dma(f32x16 (&acc)[2][4], const DmaLoader<NG> &ld, char *lds,
+                                                   int n_slabs, const int (&wrow)[2], int lane, int grp,
+                                                   const uint8_t *tok_sc_base, const uint32_t (&tok_sc)[4],
+                                                   const uint8_t *w_sc_base, const uint32_t (&w_sc)[2]) {
+    using G = Geo<NG>;
+    ld.issue(lds, 0);
+    uint32_t stok[4] = {0, 0, 0, 0}, sw[2] = {0, 0};
+    uint32_t ntok[4] = {0, 0, 0, 0}, nw[2] = {0, 0};
+    if constexpr (DT == DT_FP8 && COMPUTE) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if (t < NTF) stok[t] = *reinterpret_cast<const uint32_t *>(tok_sc_base + tok_sc[t]);
+#pragma unroll
+        for (int f = 0; f < 2; ++f) sw[f] = *reinterpret_cast<const uint32_t *>(w_sc_base + w_sc[f]);
+    }
+    FragsBf16 fx, fy;  // fy carries the held-back sub-step across the barrier
+    if constexpr (DT == DT_BF16 && COMPUTE) {
+#pragma unroll
+        for (int f = 0; f < 2; ++f)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) fy.a[f][i] = (__bf16)0.0f;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) fy.b[t][i] = (__bf16)0.0f;
+    }
+    DmaLoader<NG>::wait_all();
+    __syncthreads();  // this wave's copies have landed; now everybody else's have too
+    // One slab: `cur` is read with ds_read while `nxt` is being filled by the copies issued here.
+    auto slab = [&](const char *cur, char *nxt, int kt) __attribute__((always_inline)) {
+        const bool more = kt + 1 < n_slabs;
+        if (more) {
+            ld.issue(nxt, (uint32_t)(kt + 1) * kRowBytes);
+            if constexpr (DT == DT_FP8 && COMPUTE) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (t < NTF) ntok[t] = *reinterpret_cast<const uint32_t *>(tok_sc_base + (tok_sc[t] + (uint32_t)(kt + 1) * 4));
+#pragma unroll
+                for (int f = 0; f < 2; ++f)
+                    nw[f] = *reinterpret_cast<const uint32_t *>(w_sc_base + (w_sc[f] + (uint32_t)(kt + 1) * 512));
+            }
+        }
+        if constexpr (COMPUTE) {
+            const char *tok = cur + grp * kGroupRegion;
+            const char *wgt = cur + G::kTokRegion;
+            if constexpr (DT == DT_BF16) {
+                fetch_bf16<NTF>(fx, tok, wgt, wrow, lane, 0);
+                mma_bf16<NTF, TRANSPOSED>(acc, fy);  // sub-step 3 of the previous slab (zeros the first time)
+                fetch_bf16<NTF>(fy, tok, wgt, wrow, lane, 1);
+                mma_bf16<NTF, TRANSPOSED>(acc, fx);
+                fetch_bf16<NTF>(fx, tok, wgt, wrow, lane, 2);
+                mma_bf16<NTF, TRANSPOSED>(acc, fy);
+                fetch_bf16<NTF>(fy, tok, wgt, wrow, lane, 3);
+                mma_bf16<NTF, TRANSPOSED>(acc, fx);
+            } else {
+                mfma_slab<DT, NTF, TRANSPOSED, false>(acc, tok, wgt, wrow, lane, stok, sw);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) stok[t] = ntok[t];
+#pragma unroll
+                for (int f = 0; f < 2; ++f) sw[f] = nw[f];
+            }
+        }
+        DmaLoader<NG>::wait_all();
+        __syncthreads();
+    };
+    char *const s0 = lds, *const s1 = lds + G::kStageBytes;
+    int kt = 0;
+    for (; kt + 1 < n_slabs; kt += 2) {
+        slab(s0, s1, kt);
+        slab(s1, s0, kt + 1);
+    }
+    if (kt < n_slabs) slab(s0, s1, kt);
+    if constexpr (DT == DT_BF16 && COMPUTE) mma_bf16<NTF, TRANSPOSED>(acc, fy);
 }
 
 __device__ __forceinline__ void zero_acc(f32x16 (&acc)[2][4]) {
@@ -161,12 +270,12 @@ __device__ __forceinline__ void zero_acc(f32x16 (&acc)[2][4]) {
             for (int i = 0; i < 16; ++i) acc[f][t][i] = 0.f;
 }
 
-// Adds w[row] * acc into accum[token, col] for the live rows of the block.  Accumulator layout
-// (tokens on the MFMA M side): register i of lane l = row 32t + 8(i/4) + 4(l/32) + i%4,
+// Adds w[row] * acc into accum[token, col] for the live rows of a group's block.  Accumulator
+// layout (tokens on the MFMA M side): register i of lane l = row 32t + 8(i/4) + 4(l/32) + i%4,
 // column col0 + 32f + l%32, so one instruction adds two 128-byte runs.
 template <int NTF>
-__device__ __forceinline__ void scatter_add(const f32x16 (&acc)[2][4], const RowInfo &ri,
-                                            float *accum, int K, int col0, int lane) {
+__device__ __forceinline__ void scatter_add(const f32x16 (&acc)[2][4], const int *row_tok,
+                                            const float *row_wt, float *accum, int K, int col0, int lane) {
     const int half = lane >> 5;
     const int c = lane & 31;
 #pragma unroll
@@ -175,8 +284,8 @@ __device__ __forceinline__ void scatter_add(const f32x16 (&acc)[2][4], const Row
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int row = 32 * t + 8 * (i >> 2) + 4 * half + (i & 3);
-                const int tok = ri.tok[row];
-                const float w = ri.wt[row];
+                const int tok = row_tok[row];
+                const float w = row_wt[row];
                 if (tok >= 0) {
 #pragma unroll
                     for (int f = 0; f < 2; ++f) {
@@ -191,129 +300,159 @@ __device__ __forceinline__ void scatter_add(const f32x16 (&acc)[2][4], const Row
 
 // ------------------------------------------------------------------------------------------
 // Up kernel (and, with FUSED, the whole split==0 pipeline).
-// Tile: row block `blk` x activation columns [128*ht, 128*ht+128).  LDS weight rows 0..127 are
-// gate rows, 128..255 the matching up rows; wave v owns gate/up rows 32v..32v+31 so gate and up
-// of one activation element sit in the same lane and register.  Weight rows go on the MFMA M
-// side: a lane then holds 16 of the 32 activation columns of one MX block of its token and
-// the block maximum needs a single cross-lane exchange.
-template <int DT, bool FUSED, int NTF>
-__device__ __forceinline__ void up_tile(const MoeArgs &a, int blk, int ht, int e, RowInfo &ri,
-                                        char *lds, char *act_lds, uint32_t *act_sc_lds) {
+// Tile: NG row blocks x activation columns [128*ht, 128*ht+128).  LDS weight rows 0..127 are
+// gate rows, 128..255 the matching up rows; wave v of a group owns gate/up rows 32v..32v+31 so
+// gate and up of one activation element sit in the same lane and register.  Weight rows go on
+// the MFMA M side: a lane then holds 16 of the 32 activation columns of one MX block of its
+// token and the block maximum needs a single cross-lane exchange.
+template <int DT, bool FUSED, int NG, int NTF>
+__device__ __forceinline__ void up_tile(const MoeArgs &a, int first, int nb, int ht, int e,
+                                        RowInfo<NG> &ri, char *lds, char *act_lds, uint32_t *act_sc_lds) {
+    using G = Geo<NG>;
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
     const int r = lane & 31, half = lane >> 5;
     const int K = a.K, H = a.H, N = a.N;
     const int h0 = ht * 128;
+    const int my_ntf = (ri.nvalid[grp] + 31) >> 5;
+    const bool active = __builtin_amdgcn_readfirstlane(my_ntf) > 0;
 
-    StageLoader ld;
+    // NG == 2: DMA copies (the lane landing in LDS slot `chunk` fetches global chunk chunk ^ swz);
+    // NG == 1: register-staged copies (the thread fetching global chunk `chunk` writes slot chunk ^ swz)
+    typename std::conditional<NG == 2, DmaLoader<NG>, StageLoader<NG>>::type ld;
     const int lrow = tid >> 3, chunk = tid & 7;
-    ld.lds_off = lrow * kRowBytes + ((chunk ^ swz(lrow)) << 4);
+    const int gchunk = NG == 2 ? (chunk ^ swz(lrow)) : chunk;
+    if constexpr (NG == 2) ld.lds_wave_off = __builtin_amdgcn_readfirstlane((tid >> 6) * 8 * kRowBytes);
+    else ld.lds_off = lrow * kRowBytes + ((chunk ^ swz(lrow)) << 4);
+    ld.tok_mask = 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        int tok = ri.tok[lrow + 32 * i];
+    for (int i = 0; i < G::kTokPasses; ++i) {
+        const int row = lrow + i * G::kPassRows;
+        int tok = ri.tok[row];
         if (tok < 0) tok = 0;
-        ld.tok_ptr[i] = a.x + (int64_t)tok * K * ES + chunk * 16;
+        ld.tok_off[i] = (uint32_t)tok * (uint32_t)(K * ES) + gchunk * 16;
+        if (((row & 127) >> 5) < ((ri.nvalid[row >> 7] + 31) >> 5)) ld.tok_mask |= 1 << i;
     }
-    ld.w_ptr[0] = a.w1 + ((int64_t)e * N + h0 + lrow) * K * ES + chunk * 16;
-    ld.w_ptr[1] = ld.w_ptr[0] + (int64_t)H * K * ES;
-    ld.w_pitch32 = (int64_t)32 * K * ES;
+    ld.tok_mask = __builtin_amdgcn_readfirstlane(ld.tok_mask);  // a wave's 8 rows share a fragment
+    ld.tok_base = a.x;
+    ld.w_base[0] = a.w1 + ((int64_t)e * N + h0) * K * ES;
+    ld.w_base[1] = ld.w_base[0] + (int64_t)H * K * ES;
+    ld.w_off = (uint32_t)lrow * (uint32_t)(K * ES) + gchunk * 16;
+    ld.w_pitch_pass = (uint32_t)G::kPassRows * (uint32_t)(K * ES);
 
-    const int wrow[2] = {32 * wave, 128 + 32 * wave};
-    const uint8_t *tok_sc[4] = {nullptr, nullptr, nullptr, nullptr};
-    const uint8_t *w_sc[2] = {nullptr, nullptr};
+    const int wrow[2] = {32 * w4, 128 + 32 * w4};
+    uint32_t tok_sc[4] = {0, 0, 0, 0}, w_sc[2] = {0, 0};
+    const uint8_t *tok_sc_base = a.x_scales, *w_sc_base = nullptr;
     if constexpr (DT == DT_FP8) {
         const int kb = K >> 5;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            int tok = ri.tok[32 * t + r];
+            int tok = ri.tok[grp * kBlockRows + 32 * t + r];
             if (tok < 0) tok = 0;
-            tok_sc[t] = a.x_scales + (int64_t)tok * kb;
+            tok_sc[t] = (uint32_t)tok * (uint32_t)kb;
         }
-        const uint8_t *eb = a.w1_scales + (int64_t)e * N * kb;
-        w_sc[0] = eb + blocked_scale_off(h0 + 32 * wave + r, 0, K >> 7);
-        w_sc[1] = eb + blocked_scale_off(H + h0 + 32 * wave + r, 0, K >> 7);
+        w_sc_base = a.w1_scales + (int64_t)e * N * kb;
+        w_sc[0] = (uint32_t)blocked_scale_off(h0 + 32 * w4 + r, 0, K >> 7);
+        w_sc[1] = (uint32_t)blocked_scale_off(H + h0 + 32 * w4 + r, 0, K >> 7);
     }
 
     f32x16 acc[2][4];
     zero_acc(acc);
-    tile_main_loop<DT, NTF, true>(acc, ld, lds, (K * ES) / kRowBytes, wrow, lane, tok_sc, w_sc);
+    if constexpr (NG == 2) {
+        if (active)
+            tile_main_loop_dma<DT, NG, NTF, true, true>(acc, ld, lds, (K * ES) / kRowBytes, wrow, lane, grp,
+                                                        tok_sc_base, tok_sc, w_sc_base, w_sc);
+        else
+            tile_main_loop_dma<DT, NG, NTF, true, false>(acc, ld, lds, (K * ES) / kRowBytes, wrow, lane, grp,
+                                                         tok_sc_base, tok_sc, w_sc_base, w_sc);
+    } else {
+        tile_main_loop<DT, NG, NTF, true, true>(acc, ld, lds, (K * ES) / kRowBytes, wrow, lane, grp, tok_sc_base,
+                                                tok_sc, w_sc_base, w_sc);
+    }
 
     // ---- epilogue: SwiGLU in registers; the 2H-wide gate/up tensor never leaves the chip ----
     // (the main loop ended with a barrier, so the stage buffers may be overwritten)
-    char *tile = FUSED ? act_lds : lds;
+    constexpr int kPitch = DT == DT_BF16 ? kActPitchBf16 : kActPitchFp8;
+    char *tile = FUSED ? act_lds : lds + grp * (kBlockRows * kPitch);
+    uint32_t *sc_tile = act_sc_lds + grp * kBlockRows;
+    if (active) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        if (t < NTF) {
-            float v[16];
+        for (int t = 0; t < 4; ++t) {
+            if (t < NTF) {
+                float v[16];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) v[i] = swiglu(acc[0][t][i], acc[1][t][i]);
-            const int row = 32 * t + r;
-            if constexpr (DT == DT_BF16) {
+                for (int i = 0; i < 16; ++i) v[i] = swiglu(acc[0][t][i], acc[1][t][i]);
+                const int row = 32 * t + r;
+                if constexpr (DT == DT_BF16) {
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int hl = 32 * wave + 8 * g + 4 * half;  // tile-local activation column
-                    uint2 pk;
-                    pk.x = f32_to_bf16_bits(v[4 * g]) | (f32_to_bf16_bits(v[4 * g + 1]) << 16);
-                    pk.y = f32_to_bf16_bits(v[4 * g + 2]) | (f32_to_bf16_bits(v[4 * g + 3]) << 16);
-                    char *dst;
-                    if constexpr (FUSED) {
-                        const int byte = (hl & 63) * 2;
-                        dst = tile + (hl >> 6) * kTokRegion + row * kRowBytes +
-                              (((byte >> 4) ^ swz(row)) << 4) + (byte & 15);
-                    } else {
-                        dst = tile + row * kActPitchBf16 + hl * 2;
+                    for (int g = 0; g < 4; ++g) {
+                        const int hl = 32 * w4 + 8 * g + 4 * half;  // tile-local activation column
+                        uint2 pk;
+                        pk.x = f32_to_bf16_bits(v[4 * g]) | (f32_to_bf16_bits(v[4 * g + 1]) << 16);
+                        pk.y = f32_to_bf16_bits(v[4 * g + 2]) | (f32_to_bf16_bits(v[4 * g + 3]) << 16);
+                        char *dst;
+                        if constexpr (FUSED) {
+                            const int byte = (hl & 63) * 2;
+                            dst = tile + (hl >> 6) * kGroupRegion + row * kRowBytes +
+                                  (((byte >> 4) ^ swz(row)) << 4) + (byte & 15);
+                        } else {
+                            dst = tile + row * kActPitchBf16 + hl * 2;
+                        }
+                        *reinterpret_cast<uint2 *>(dst) = pk;
                     }
-                    *reinterpret_cast<uint2 *>(dst) = pk;
-                }
-            } else {
-                float amax = 0.f;
+                } else {
+                    float amax = 0.f;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(v[i]));
-                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-                uint32_t e8;
-                float inv;
-                mx_block_scale(amax, e8, inv);
+                    for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(v[i]));
+                    amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+                    uint32_t e8;
+                    float inv;
+                    mx_block_scale(amax, e8, inv);
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int hl = 32 * wave + 8 * g + 4 * half;
-                    const uint32_t q = pack4_e4m3(v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3], inv);
-                    char *dst;
-                    if constexpr (FUSED)
-                        dst = tile + row * kRowBytes + (((hl >> 4) ^ swz(row)) << 4) + (hl & 15);
-                    else
-                        dst = tile + row * kActPitchFp8 + hl;
-                    *reinterpret_cast<uint32_t *>(dst) = q;
+                    for (int g = 0; g < 4; ++g) {
+                        const int hl = 32 * w4 + 8 * g + 4 * half;
+                        const uint32_t q = pack4_e4m3(v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3], inv);
+                        char *dst;
+                        if constexpr (FUSED)
+                            dst = tile + row * kRowBytes + (((hl >> 4) ^ swz(row)) << 4) + (hl & 15);
+                        else
+                            dst = tile + row * kActPitchFp8 + hl;
+                        *reinterpret_cast<uint32_t *>(dst) = q;
+                    }
+                    if (half == 0) reinterpret_cast<uint8_t *>(sc_tile)[row * 4 + w4] = (uint8_t)e8;
                 }
-                if (half == 0) reinterpret_cast<uint8_t *>(act_sc_lds)[row * 4 + wave] = (uint8_t)e8;
             }
         }
     }
     __syncthreads();
     if constexpr (!FUSED) {
-        // coalesced copy of the live rows of the tile to the activation workspace
-        const int64_t row0 = (int64_t)blk * kTokRows;
-        if constexpr (DT == DT_BF16) {
-            const int c = tid & 15;
+        // coalesced copy of the live rows of the group's tile to the activation workspace
+        if (active) {
+            const int64_t row0 = (int64_t)(first + grp) * kBlockRows;
+            if constexpr (DT == DT_BF16) {
+                const int c = gt & 15;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int row = (tid >> 4) + 16 * i;
-                if (row < 32 * NTF) {
-                    uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchBf16 + c * 16);
-                    *reinterpret_cast<uint4 *>(a.act + ((row0 + row) * H + h0) * 2 + c * 16) = v;
+                for (int i = 0; i < 8; ++i) {
+                    const int row = (gt >> 4) + 16 * i;
+                    if (row < 32 * my_ntf) {
+                        uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchBf16 + c * 16);
+                        *reinterpret_cast<uint4 *>(a.act + ((row0 + row) * H + h0) * 2 + c * 16) = v;
+                    }
                 }
-            }
-        } else {
-            const int c = tid & 7;
+            } else {
+                const int c = gt & 7;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int row = (tid >> 3) + 32 * i;
-                if (i < NTF) {
-                    uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchFp8 + c * 16);
-                    *reinterpret_cast<uint4 *>(a.act + (row0 + row) * H + h0 + c * 16) = v;
+                for (int i = 0; i < 4; ++i) {
+                    const int row = (gt >> 3) + 32 * i;
+                    if (i < my_ntf) {
+                        uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchFp8 + c * 16);
+                        *reinterpret_cast<uint4 *>(a.act + (row0 + row) * H + h0 + c * 16) = v;
+                    }
                 }
+                if (gt < 32 * my_ntf)
+                    *reinterpret_cast<uint32_t *>(a.act_scales + (row0 + gt) * (H >> 5) + ht * 4) = sc_tile[gt];
             }
-            if (tid < 32 * NTF)
-                *reinterpret_cast<uint32_t *>(a.act_scales + (row0 + tid) * (H >> 5) + ht * 4) = act_sc_lds[tid];
         }
     }
 }
@@ -321,9 +460,10 @@ __device__ __forceinline__ void up_tile(const MoeArgs &a, int blk, int ht, int e
 // Down phase of the split==0 pipeline: the activation tile (128 rows x 128 columns of H) stays in
 // LDS as the token operand; W2[e][256-row chunk][h-slice] streams through the weight region.
 template <int DT, int NTF>
-__device__ __forceinline__ void fused_down_phase(const MoeArgs &a, int ht, int e, RowInfo &ri,
+__device__ __forceinline__ void fused_down_phase(const MoeArgs &a, int ht, int e, RowInfo<1> &ri,
                                                  char *lds, const char *act_lds,
                                                  const uint32_t *act_sc_lds) {
+    using G = Geo<1>;
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
     constexpr int NS = DT == DT_BF16 ? 2 : 1;  // 128-byte slabs across the 128-column h-slice
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -332,15 +472,17 @@ __device__ __forceinline__ void fused_down_phase(const MoeArgs &a, int ht, int e
     const int n_chunks = (K + kWRows - 1) / kWRows;
     const int n_steps = n_chunks * NS;
 
-    StageLoader ld;
+    StageLoader<1> ld;
     const int lrow = tid >> 3, chunk = tid & 7;
     ld.lds_off = lrow * kRowBytes + ((chunk ^ swz(lrow)) << 4);
-    ld.w_pitch32 = (int64_t)32 * H * ES;
-    const char *w2e = a.w2 + (int64_t)e * K * H * ES + (int64_t)ht * 128 * ES + chunk * 16;
+    ld.tok_mask = 0;
+    ld.w_pitch_pass = (uint32_t)G::kPassRows * (uint32_t)(H * ES);
+    ld.w_off = (uint32_t)lrow * (uint32_t)(H * ES) + chunk * 16;
+    const char *w2e = a.w2 + (int64_t)e * K * H * ES + (int64_t)ht * 128 * ES;
     auto set_chunk = [&](int kc) {
         const int k0 = kc * kWRows;
-        ld.w_ptr[0] = w2e + (int64_t)(k0 + lrow) * H * ES;
-        ld.w_ptr[1] = (k0 + 128 < K) ? ld.w_ptr[0] + (int64_t)128 * H * ES : ld.w_ptr[0];
+        ld.w_base[0] = w2e + (int64_t)k0 * H * ES;
+        ld.w_base[1] = (k0 + 128 < K) ? ld.w_base[0] + (int64_t)128 * H * ES : ld.w_base[0];
     };
     const int wrow[2] = {64 * wave, 64 * wave + 32};
     uint32_t stok[4] = {0, 0, 0, 0}, sw[2] = {0, 0};
@@ -369,111 +511,184 @@ __device__ __forceinline__ void fused_down_phase(const MoeArgs &a, int ht, int e
     __syncthreads();
     for (int s = 0; s < n_steps; ++s) {
         const int kc = s / NS, sl = s - kc * NS;
-        char *cur = lds + (s & 1) * kStageBytes;
-        char *nxt = lds + ((s + 1) & 1) * kStageBytes;
+        char *cur = lds + (s & 1) * G::kStageBytes;
+        char *nxt = lds + ((s + 1) & 1) * G::kStageBytes;
         const bool more = s + 1 < n_steps;
         if (more) {
             const int nkc = (s + 1) / NS, nsl = (s + 1) - nkc * NS;
             if (nsl == 0) set_chunk(nkc);
-            ld.load_w((int64_t)nsl * kRowBytes);
+            ld.load_w((uint32_t)nsl * kRowBytes);
         }
         if (sl == 0) {
             zero_acc(acc);
             load_wscales(kc);
         }
-        mfma_slab<DT, NTF, false>(acc, act_lds + sl * kTokRegion, cur + kTokRegion, wrow, lane, stok, sw);
-        if (sl == NS - 1) scatter_add<NTF>(acc, ri, a.accum, K, kc * kWRows + 64 * wave, lane);
+        mfma_slab<DT, NTF, false, true>(acc, act_lds + sl * kGroupRegion, cur + G::kTokRegion, wrow, lane, stok, sw);
+        if (sl == NS - 1) scatter_add<NTF>(acc, ri.tok, ri.wt, a.accum, K, kc * kWRows + 64 * wave, lane);
         if (more) ld.store_w(nxt);
         __syncthreads();
     }
 }
 
-template <int DT, bool FUSED>
-__global__ __launch_bounds__(kThreads) void moe_up_kernel(MoeArgs a) {
-    __shared__ __attribute__((aligned(1024))) char lds[kNumStages * kStageBytes];
-    __shared__ __attribute__((aligned(1024))) char act_lds[FUSED ? (DT == DT_BF16 ? 2 : 1) * kTokRegion : 16];
-    __shared__ uint32_t act_sc_lds[kTokRows];
-    __shared__ RowInfo ri;
-    int blk, ht;
-    if (!map_tile(a, blk, ht)) return;
-    if (blk * kTokRows >= a.ntpp[0]) return;
-    const int ntf = load_row_info(a, blk, ri);
+template <int DT, bool FUSED, int NG>
+__global__ __launch_bounds__(256 * NG) void moe_up_kernel(MoeArgs a) {
+    static_assert(!FUSED || NG == 1, "the fused pipeline keeps one row block per workgroup");
+    __shared__ __attribute__((aligned(1024))) char lds[kNumStages * Geo<NG>::kStageBytes];
+    __shared__ __attribute__((aligned(1024))) char act_lds[FUSED ? (DT == DT_BF16 ? 2 : 1) * kGroupRegion : 16];
+    __shared__ uint32_t act_sc_lds[kBlockRows * NG];
+    __shared__ RowInfo<NG> ri;
+    int first, nb, ht;
+    if (!resolve_tile<NG>(a, first, nb, ht)) return;
+    if (first * kBlockRows >= a.ntpp[0]) return;
+    const int ntf = load_row_info<NG>(a, first, nb, ri);
     if (ntf == 0) return;
-    const int e = a.expert_ids[blk];
+    const int e = a.expert_ids[first];
     if (e < 0 || e >= a.E) return;
     if (ntf == 1) {
-        up_tile<DT, FUSED, 1>(a, blk, ht, e, ri, lds, act_lds, act_sc_lds);
+        up_tile<DT, FUSED, NG, 1>(a, first, nb, ht, e, ri, lds, act_lds, act_sc_lds);
         if constexpr (FUSED) fused_down_phase<DT, 1>(a, ht, e, ri, lds, act_lds, act_sc_lds);
     } else if (ntf == 2) {
-        up_tile<DT, FUSED, 2>(a, blk, ht, e, ri, lds, act_lds, act_sc_lds);
+        up_tile<DT, FUSED, NG, 2>(a, first, nb, ht, e, ri, lds, act_lds, act_sc_lds);
         if constexpr (FUSED) fused_down_phase<DT, 2>(a, ht, e, ri, lds, act_lds, act_sc_lds);
     } else {
-        up_tile<DT, FUSED, 4>(a, blk, ht, e, ri, lds, act_lds, act_sc_lds);
+        up_tile<DT, FUSED, NG, 4>(a, first, nb, ht, e, ri, lds, act_lds, act_sc_lds);
         if constexpr (FUSED) fused_down_phase<DT, 4>(a, ht, e, ri, lds, act_lds, act_sc_lds);
     }
 }
 
-// Down kernel of the split pipeline: y[128 rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
+// Down kernel of the split pipeline: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
 // full reduction over H inside the workgroup (no split-K), then w[row] * y added to accum[token].
-template <int DT, int NTF>
-__device__ __forceinline__ void down_tile(const MoeArgs &a, int blk, int kt, int e, RowInfo &ri, char *lds) {
+template <int DT, int NG, int NTF>
+__device__ __forceinline__ void down_tile(const MoeArgs &a, int first, int kt, int e, RowInfo<NG> &ri, char *lds) {
+    using G = Geo<NG>;
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int grp = wave >> 2, w4 = wave & 3;
     const int r = lane & 31;
     const int K = a.K, H = a.H;
     const int k0 = kt * kWRows;
-    const int64_t row0 = (int64_t)blk * kTokRows;
+    const int64_t row0 = (int64_t)first * kBlockRows;
+    const bool active = __builtin_amdgcn_readfirstlane(ri.nvalid[grp]) > 0;
 
-    StageLoader ld;
+    typename std::conditional<NG == 2, DmaLoader<NG>, StageLoader<NG>>::type ld;
     const int lrow = tid >> 3, chunk = tid & 7;
-    ld.lds_off = lrow * kRowBytes + ((chunk ^ swz(lrow)) << 4);
+    const int gchunk = NG == 2 ? (chunk ^ swz(lrow)) : chunk;
+    if constexpr (NG == 2) ld.lds_wave_off = __builtin_amdgcn_readfirstlane((tid >> 6) * 8 * kRowBytes);
+    else ld.lds_off = lrow * kRowBytes + ((chunk ^ swz(lrow)) << 4);
+    ld.tok_mask = 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-        ld.tok_ptr[i] = a.act + (row0 + lrow + 32 * i) * H * ES + chunk * 16;
-    ld.w_ptr[0] = a.w2 + ((int64_t)e * K + k0 + lrow) * H * ES + chunk * 16;
-    ld.w_ptr[1] = (k0 + 128 < K) ? ld.w_ptr[0] + (int64_t)128 * H * ES : ld.w_ptr[0];
-    ld.w_pitch32 = (int64_t)32 * H * ES;
+    for (int i = 0; i < G::kTokPasses; ++i) {
+        const int row = lrow + i * G::kPassRows;
+        ld.tok_off[i] = (uint32_t)row * (uint32_t)(H * ES) + gchunk * 16;
+        if (((row & 127) >> 5) < ((ri.nvalid[row >> 7] + 31) >> 5)) ld.tok_mask |= 1 << i;
+    }
+    ld.tok_mask = __builtin_amdgcn_readfirstlane(ld.tok_mask);  // a wave's 8 rows share a fragment
+    ld.tok_base = a.act + row0 * H * ES;
+    ld.w_base[0] = a.w2 + ((int64_t)e * K + k0) * H * ES;
+    ld.w_base[1] = (k0 + 128 < K) ? ld.w_base[0] + (int64_t)128 * H * ES : ld.w_base[0];
+    ld.w_off = (uint32_t)lrow * (uint32_t)(H * ES) + gchunk * 16;
+    ld.w_pitch_pass = (uint32_t)G::kPassRows * (uint32_t)(H * ES);
 
-    const int wrow[2] = {64 * wave, 64 * wave + 32};
-    const uint8_t *tok_sc[4] = {nullptr, nullptr, nullptr, nullptr};
-    const uint8_t *w_sc[2] = {nullptr, nullptr};
+    const int wrow[2] = {64 * w4, 64 * w4 + 32};
+    uint32_t tok_sc[4] = {0, 0, 0, 0}, w_sc[2] = {0, 0};
+    const uint8_t *tok_sc_base = nullptr, *w_sc_base = nullptr;
     if constexpr (DT == DT_FP8) {
+        tok_sc_base = a.act_scales + row0 * (H >> 5);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) tok_sc[t] = a.act_scales + (row0 + 32 * t + r) * (H >> 5);
-        const uint8_t *eb = a.w2_scales + (int64_t)e * K * (H >> 5);
+        for (int t = 0; t < 4; ++t) tok_sc[t] = (uint32_t)(grp * kBlockRows + 32 * t + r) * (uint32_t)(H >> 5);
+        w_sc_base = a.w2_scales + (int64_t)e * K * (H >> 5);
 #pragma unroll
         for (int f = 0; f < 2; ++f) {
-            int row = k0 + 64 * wave + 32 * f + r;
+            int row = k0 + 64 * w4 + 32 * f + r;
             if (row >= K) row = K - 1;
-            w_sc[f] = eb + blocked_scale_off(row, 0, H >> 7);
+            w_sc[f] = (uint32_t)blocked_scale_off(row, 0, H >> 7);
         }
     }
     f32x16 acc[2][4];
     zero_acc(acc);
-    tile_main_loop<DT, NTF, false>(acc, ld, lds, (H * ES) / kRowBytes, wrow, lane, tok_sc, w_sc);
-    scatter_add<NTF>(acc, ri, a.accum, K, k0 + 64 * wave, lane);
+    if constexpr (NG == 2) {
+        if (active)
+            tile_main_loop_dma<DT, NG, NTF, false, true>(acc, ld, lds, (H * ES) / kRowBytes, wrow, lane, grp,
+                                                         tok_sc_base, tok_sc, w_sc_base, w_sc);
+        else
+            tile_main_loop_dma<DT, NG, NTF, false, false>(acc, ld, lds, (H * ES) / kRowBytes, wrow, lane, grp,
+                                                          tok_sc_base, tok_sc, w_sc_base, w_sc);
+    } else {
+        tile_main_loop<DT, NG, NTF, false, true>(acc, ld, lds, (H * ES) / kRowBytes, wrow, lane, grp, tok_sc_base,
+                                                 tok_sc, w_sc_base, w_sc);
+    }
+    if (active)
+        scatter_add<NTF>(acc, ri.tok + grp * kBlockRows, ri.wt + grp * kBlockRows, a.accum, K, k0 + 64 * w4, lane);
 }
 
-template <int DT>
-__global__ __launch_bounds__(kThreads) void moe_down_kernel(MoeArgs a) {
-    __shared__ __attribute__((aligned(1024))) char lds[kNumStages * kStageBytes];
-    __shared__ RowInfo ri;
-    int blk, kt;
-    if (!map_tile(a, blk, kt)) return;
-    if (blk * kTokRows >= a.ntpp[0]) return;
-    const int ntf = load_row_info(a, blk, ri);
+template <int DT, int NG>
+__global__ __launch_bounds__(256 * NG) void moe_down_kernel(MoeArgs a) {
+    __shared__ __attribute__((aligned(1024))) char lds[kNumStages * Geo<NG>::kStageBytes];
+    __shared__ RowInfo<NG> ri;
+    int first, nb, kt;
+    if (!resolve_tile<NG>(a, first, nb, kt)) return;
+    if (first * kBlockRows >= a.ntpp[0]) return;
+    const int ntf = load_row_info<NG>(a, first, nb, ri);
     if (ntf == 0) return;
-    const int e = a.expert_ids[blk];
+    const int e = a.expert_ids[first];
     if (e < 0 || e >= a.E) return;
-    if (ntf == 1) down_tile<DT, 1>(a, blk, kt, e, ri, lds);
-    else if (ntf == 2) down_tile<DT, 2>(a, blk, kt, e, ri, lds);
-    else down_tile<DT, 4>(a, blk, kt, e, ri, lds);
+    if (ntf == 1) down_tile<DT, NG, 1>(a, first, kt, e, ri, lds);
+    else if (ntf == 2) down_tile<DT, NG, 2>(a, first, kt, e, ri, lds);
+    else down_tile<DT, NG, 4>(a, first, kt, e, ri, lds);
 }
 
-__global__ __launch_bounds__(256) void zero_f32_kernel(float4 *p, int64_t n4) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride)
-        p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+// Prologue of every call: clears the fp32 accumulator and (workgroup 0) builds the list of row
+// tiles for the two-group kernels: consecutive blocks of one expert are paired, an expert's odd
+// last block stays single.  One pass of block-wide scans per 256 blocks.
+__global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert_ids, const int32_t *ntpp,
+                                                           int n_blocks, int2 *tiles, int *n_tiles,
+                                                           float4 *accum, int64_t n4, int do_zero) {
+    if (blockIdx.x == 0 && tiles != nullptr) {
+        __shared__ int s_max[4], s_sum[4], s_carry[2];
+        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        const int n_live = min((ntpp[0] + kBlockRows - 1) / kBlockRows, n_blocks);
+        if (tid == 0) { s_carry[0] = 0; s_carry[1] = 0; }
+        __syncthreads();
+        for (int base = 0; base < n_live; base += 256) {
+            const int b = base + tid;
+            const bool live = b < n_live;
+            const int e = live ? expert_ids[b] : -2;
+            const int prev = (live && b > 0) ? expert_ids[b - 1] : -1;
+            int v = (live && e != prev) ? b : -1;  // start of a run of equal experts
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int t = __shfl_up(v, d, 64);
+                if (lane >= d) v = max(v, t);
+            }
+            if (lane == 63) s_max[wave] = v;
+            __syncthreads();
+            int run_start = s_carry[0];
+            for (int w = 0; w < wave; ++w) run_start = max(run_start, s_max[w]);
+            run_start = max(run_start, v);
+            const bool leader = live && (((b - run_start) & 1) == 0);
+            const bool paired = leader && (b + 1 < n_live) && expert_ids[b + 1] == e;
+            int incl = leader ? 1 : 0;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int t = __shfl_up(incl, d, 64);
+                if (lane >= d) incl += t;
+            }
+            if (lane == 63) s_sum[wave] = incl;
+            __syncthreads();
+            int off = s_carry[1];
+            for (int w = 0; w < wave; ++w) off += s_sum[w];
+            if (leader) tiles[off + incl - 1] = make_int2(b, paired ? 2 : 1);
+            __syncthreads();
+            if (tid == 255) { s_carry[0] = run_start; s_carry[1] = off + incl; }
+            __syncthreads();
+        }
+        if (tid == 0) n_tiles[0] = s_carry[1];
+    }
+    if (do_zero) {
+        const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+        for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride)
+            accum[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
 }
 
 // out = bf16(accum)  (ACCUMULATE: out = bf16(float(out) + accum)); 8 elements per thread step.
@@ -502,14 +717,18 @@ __global__ __launch_bounds__(256) void finalize_kernel(const float4 *acc, uint4 
 // ------------------------------------------------------------------------------------------ host
 
 struct WorkspaceLayout {
-    size_t accum_off, act_off, act_scales_off, total;
+    size_t n_tiles_off, tiles_off, accum_off, act_off, act_scales_off, total;
 };
 
 static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_num, int split) {
     WorkspaceLayout l{};
     const size_t H = (size_t)N / 2;
-    const size_t rows = align_up((size_t)sorted_num, kTokRows);
+    const size_t rows = align_up((size_t)sorted_num, kBlockRows);
     size_t off = 0;
+    l.n_tiles_off = off;
+    off += 256;
+    l.tiles_off = off;
+    off = align_up(off + (rows / kBlockRows) * sizeof(int2), 256);
     l.accum_off = off;
     off = align_up(off + (size_t)M * K * sizeof(float), 256);
     l.act_off = off;
@@ -533,24 +752,28 @@ template <int DT>
 static int launch_pipeline(MoeArgs a, void *out, int split, hipStream_t s) {
     const int64_t n_out = (int64_t)a.M * a.K;  // K % 128 == 0, so n_out % 8 == 0
     const int mask = g_phase_mask;
-    if (mask & PMOE_PHASE_ZERO) {
-        const int64_t n4 = n_out / 4;
-        const int blocks = (int)std::min<int64_t>((n4 + 255) / 256, 2048);
-        hipLaunchKernelGGL(zero_f32_kernel, dim3(blocks), dim3(256), 0, s, reinterpret_cast<float4 *>(a.accum), n4);
-    }
-    a.n_blocks = (a.sorted_num + kTokRows - 1) / kTokRows;
+    a.n_blocks = (a.sorted_num + kBlockRows - 1) / kBlockRows;
     a.n_wtiles = a.H / 128;
+    {
+        // the tile list is needed by the two-group kernels even when the clear is masked off
+        const int64_t n4 = n_out / 4;
+        const int do_zero = (mask & PMOE_PHASE_ZERO) ? 1 : 0;
+        const int blocks = do_zero ? (int)std::min<int64_t>((n4 + 255) / 256, 2048) : 1;
+        hipLaunchKernelGGL(moe_prologue_kernel, dim3(blocks), dim3(256), 0, s, a.expert_ids, a.ntpp, a.n_blocks,
+                           split ? const_cast<int2 *>(a.tiles) : nullptr, const_cast<int *>(a.n_tiles),
+                           reinterpret_cast<float4 *>(a.accum), n4, do_zero);
+    }
     if (a.n_blocks > 0) {
         const int grid = grid_for(a.n_blocks * a.n_wtiles);
         if (split) {
             if (mask & PMOE_PHASE_UP)
-                hipLaunchKernelGGL((moe_up_kernel<DT, false>), dim3(grid), dim3(kThreads), 0, s, a);
+                hipLaunchKernelGGL((moe_up_kernel<DT, false, 2>), dim3(grid), dim3(512), 0, s, a);
             MoeArgs d = a;
             d.n_wtiles = (a.K + kWRows - 1) / kWRows;
             if (mask & PMOE_PHASE_DOWN)
-                hipLaunchKernelGGL((moe_down_kernel<DT>), dim3(grid_for(d.n_blocks * d.n_wtiles)), dim3(kThreads), 0, s, d);
+                hipLaunchKernelGGL((moe_down_kernel<DT, 2>), dim3(grid_for(d.n_blocks * d.n_wtiles)), dim3(512), 0, s, d);
         } else if (mask & PMOE_PHASE_UP) {
-            hipLaunchKernelGGL((moe_up_kernel<DT, true>), dim3(grid), dim3(kThreads), 0, s, a);
+            hipLaunchKernelGGL((moe_up_kernel<DT, true, 1>), dim3(grid), dim3(256), 0, s, a);
         }
     }
     if (mask & PMOE_PHASE_FINALIZE) {
@@ -622,6 +845,8 @@ extern "C" int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2,
     a.ntpp = num_tokens_post_padded;
     a.topk_w = topk_weights;
     char *ws = static_cast<char *>(workspace);
+    a.n_tiles = reinterpret_cast<const int *>(ws + l.n_tiles_off);
+    a.tiles = reinterpret_cast<const int2 *>(ws + l.tiles_off);
     a.accum = reinterpret_cast<float *>(ws + l.accum_off);
     a.act = ws + l.act_off;
     a.top_k = top_k; a.M = M; a.K = K; a.N = N; a.H = N / 2; a.E = num_experts; a.sorted_num = sorted_num;
@@ -660,6 +885,8 @@ extern "C" int pmoe_fused_moe_mxfp8(const void *x, const void *x_scales, const v
     a.ntpp = num_tokens_post_padded;
     a.topk_w = topk_weights;
     char *ws = static_cast<char *>(workspace);
+    a.n_tiles = reinterpret_cast<const int *>(ws + l.n_tiles_off);
+    a.tiles = reinterpret_cast<const int2 *>(ws + l.tiles_off);
     a.accum = reinterpret_cast<float *>(ws + l.accum_off);
     a.act = ws + l.act_off;
     a.act_scales = reinterpret_cast<uint8_t *>(ws + l.act_scales_off);

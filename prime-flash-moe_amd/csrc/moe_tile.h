@@ -1,15 +1,20 @@
 // Device-side tile engine shared by the fused-MoE kernels (gfx950, wave64).
 //
-// One workgroup = 256 threads = 4 waves and owns a (128 sorted rows) x (256 weight rows)
-// tile of a grouped GEMM whose two operands are both contiguous along the contraction
-// dimension:  token rows (x or the activation) and weight rows (W1 or W2 of one expert).
+// A workgroup of NG*256 threads (NG = 1 or 2 "token groups" of 4 waves) owns a tile of a grouped
+// GEMM whose two operands are both contiguous along the contraction dimension:
+//     NG*128 token rows (x or the activation; one 128-row sorted block per group)
+//   x 256 weight rows   (W1 or W2 of one expert, shared by the groups).
 // The contraction is consumed in slabs of 128 bytes per row (64 bf16 or 128 e4m3), staged
 // through LDS with a double buffer: while the MFMAs of slab k run out of one buffer, the
-// global loads of slab k+1 are in flight into registers and are written to the other buffer.
+// global loads of slab k+1 are in flight into registers and are then written to the other.
+// With NG = 2 the two groups are two waves per SIMD working on different token rows against the
+// same weight rows: the weight slab is fetched once for 256 token rows, and one group's MFMAs
+// cover the other's LDS and barrier latencies.
 //
-// LDS layout of one stage: [384 rows][128 B]; rows 0..127 token rows, 128..383 weight rows.
+// LDS layout of one stage: [NG*128 token rows][128 B] then [256 weight rows][128 B].
 // A row is 8 chunks of 16 B; chunk c of row r is stored in slot c ^ ((r >> 1) & 7), which
-// makes the 16-byte MFMA operand reads of 16 consecutive rows hit all 64 banks once.
+// makes the 16-byte MFMA operand reads of 16 consecutive rows hit all 64 banks once
+// (measured: 242 of 256 B/clk/CU, against 43 B/clk unswizzled).
 //
 // MFMA shapes: v_mfma_f32_32x32x16_bf16 (4 per slab) and v_mfma_scale_f32_32x32x64_f8f6f4
 // (2 per slab, e4m3 operands, e8m0 scales: lane l supplies the scale of (row l%32, K block l/32)).
@@ -26,13 +31,23 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kThreads = 256;
-constexpr int kTokRows = 128;   // sorted rows per block (= block_m)
-constexpr int kWRows = 256;     // weight rows per tile
-constexpr int kRowBytes = 128;  // contraction bytes per LDS row
-constexpr int kTokRegion = kTokRows * kRowBytes;             // 16 KB
-constexpr int kStageBytes = (kTokRows + kWRows) * kRowBytes;  // 48 KB
+constexpr int kBlockRows = 128;  // sorted rows per block (= block_m)
+constexpr int kWRows = 256;      // weight rows per tile
+constexpr int kRowBytes = 128;   // contraction bytes per LDS row
+constexpr int kGroupRegion = kBlockRows * kRowBytes;  // 16 KB: one group's token rows of a stage
 constexpr int kNumStages = 2;
+
+template <int NG>
+struct Geo {
+    static constexpr int kThreads = 256 * NG;
+    static constexpr int kTokRows = kBlockRows * NG;
+    static constexpr int kPassRows = 32 * NG;            // rows the workgroup moves per pass (8 threads a row)
+    static constexpr int kTokPasses = kTokRows / kPassRows;  // 4
+    static constexpr int kWPasses = kWRows / kPassRows;      // 8 or 4
+    static constexpr int kWPassesPerHalf = 128 / kPassRows;  // passes per 128 weight rows
+    static constexpr int kTokRegion = kTokRows * kRowBytes;
+    static constexpr int kStageBytes = kTokRegion + kWRows * kRowBytes;  // 48 KB or 64 KB
+};
 
 enum : int { DT_BF16 = 0, DT_FP8 = 1 };
 
@@ -80,54 +95,126 @@ __device__ __forceinline__ int64_t blocked_scale_off(int row, int kt, int n_ktil
 
 // ------------------------------------------------------------------------------------------
 // Per-thread description of the global -> LDS copy of one stage.
-// Thread t moves chunk (t & 7) of rows (t >> 3) + 32*i : i < 4 token rows, i < 8 weight rows.
+// Thread t moves chunk (t & 7) of rows (t >> 3) + kPassRows*i, for the token passes whose bit is
+// set in tok_mask and for all weight passes.
+template <int NG>
 struct StageLoader {
-    const char *tok_ptr[4];  // row start + chunk offset, per token row of this thread
-    const char *w_ptr[2];    // first / second 128 weight rows: row (t>>3) start + chunk offset
-    int64_t w_pitch32;       // bytes between weight rows 32 apart
-    int lds_off;             // byte offset of this thread's chunk inside a 32-row group
-    uint4 rt[4];
-    uint4 rw[8];
+    using G = Geo<NG>;
+    // Addresses are a workgroup-uniform base (held in scalar registers) plus a 32-bit per-thread
+    // byte offset: the token matrix and one expert's weight matrix are each below 4 GiB.
+    const char *tok_base;
+    const char *w_base[2];          // first / second 128 weight rows of the tile
+    uint32_t tok_off[G::kTokPasses];  // row start + chunk offset of this thread's token rows
+    uint32_t w_off;                  // row (t >> 3) start + chunk offset inside a 128-row half
+    uint32_t w_pitch_pass;           // bytes between weight rows kPassRows apart
+    int lds_off;                     // byte offset of this thread's chunk inside a pass
+    int tok_mask;                    // token passes that hold live rows
+    uint4 rt[G::kTokPasses];
+    uint4 rw[G::kWPasses];
 
-    template <int NTF>
-    __device__ __forceinline__ void load(int64_t koff) {
+    __device__ __forceinline__ void load_tok(uint32_t koff) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (i < NTF) rt[i] = *reinterpret_cast<const uint4 *>(tok_ptr[i] + koff);
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            rw[i] = *reinterpret_cast<const uint4 *>(w_ptr[i >> 2] + (i & 3) * w_pitch32 + koff);
+        for (int i = 0; i < G::kTokPasses; ++i)
+            if (tok_mask & (1 << i)) rt[i] = *reinterpret_cast<const uint4 *>(tok_base + (tok_off[i] + koff));
     }
-    template <int NTF>
-    __device__ __forceinline__ void load_tok(int64_t koff) {
+    __device__ __forceinline__ void load_w(uint32_t koff) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (i < NTF) rt[i] = *reinterpret_cast<const uint4 *>(tok_ptr[i] + koff);
+        for (int i = 0; i < G::kWPasses; ++i)
+            rw[i] = *reinterpret_cast<const uint4 *>(w_base[i / G::kWPassesPerHalf] +
+                                                     (w_off + (i % G::kWPassesPerHalf) * w_pitch_pass + koff));
     }
-    __device__ __forceinline__ void load_w(int64_t koff) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            rw[i] = *reinterpret_cast<const uint4 *>(w_ptr[i >> 2] + (i & 3) * w_pitch32 + koff);
-    }
-    template <int NTF>
     __device__ __forceinline__ void store_tok(char *stage) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (i < NTF) *reinterpret_cast<uint4 *>(stage + lds_off + i * 32 * kRowBytes) = rt[i];
+        for (int i = 0; i < G::kTokPasses; ++i)
+            if (tok_mask & (1 << i))
+                *reinterpret_cast<uint4 *>(stage + lds_off + i * G::kPassRows * kRowBytes) = rt[i];
     }
     __device__ __forceinline__ void store_w(char *stage) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            *reinterpret_cast<uint4 *>(stage + kTokRegion + lds_off + i * 32 * kRowBytes) = rw[i];
+        for (int i = 0; i < G::kWPasses; ++i)
+            *reinterpret_cast<uint4 *>(stage + G::kTokRegion + lds_off + i * G::kPassRows * kRowBytes) = rw[i];
     }
 };
 
 // ------------------------------------------------------------------------------------------
-// MFMA over one 128-byte slab.  `tok` / `wgt` point at the token / weight regions of a stage.
-// wrow[f] = first LDS weight row of this wave's fragment f.  TRANSPOSED: weight rows on the
-// MFMA M side (accumulator registers run along weight rows, lanes along tokens); otherwise
-// tokens on the M side (lanes run along weight rows).
-template <int DT, int NTF, bool TRANSPOSED>
+// Direct global -> LDS copy of one stage (global_load_lds_dwordx4): no staging registers and no
+// ds_write instructions.  A wave instruction moves 64 x 16 B = 8 consecutive LDS rows; lane l
+// writes LDS bytes [16 l, 16 l + 16) behind the wave-uniform base (M0), so the swizzle is applied
+// on the global side: the lane that lands in slot s of row r fetches chunk s ^ swz(r).
+template <int NG>
+struct DmaLoader {
+    using G = Geo<NG>;
+    const char *tok_base;
+    const char *w_base[2];
+    uint32_t tok_off[G::kTokPasses];
+    uint32_t w_off;
+    uint32_t w_pitch_pass;
+    int lds_wave_off;  // byte offset of this wave's 8 rows inside a pass (wave-uniform)
+    int tok_mask;      // token passes that hold live rows (wave-uniform)
+
+    // The copy is written as inline assembly: issued through the compiler's builtin, every later LDS
+    // read would first wait for all copies in flight (the compiler cannot tell the stage being read
+    // from the stage being filled), which would serialise copy and compute.  The hardware counter
+    // still counts these loads; wait_all() must run before the barrier that publishes a stage.
+    static __device__ __forceinline__ void copy16(const char *base, uint32_t voff, char *lds_dst) {
+        const uint32_t m0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)lds_dst;
+        asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :
+                     : "v"(voff), "s"(base), "s"(m0)
+                     : "memory");
+    }
+    static __device__ __forceinline__ void wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+    __device__ __forceinline__ void issue(char *stage, uint32_t koff) const {
+#pragma unroll
+        for (int i = 0; i < G::kTokPasses; ++i)
+            if (tok_mask & (1 << i))
+                copy16(tok_base, tok_off[i] + koff, stage + lds_wave_off + i * G::kPassRows * kRowBytes);
+#pragma unroll
+        for (int i = 0; i < G::kWPasses; ++i)
+            copy16(w_base[i / G::kWPassesPerHalf], w_off + (i % G::kWPassesPerHalf) * w_pitch_pass + koff,
+                   stage + G::kTokRegion + lds_wave_off + i * G::kPassRows * kRowBytes);
+    }
+};
+
+// bf16 operand fragments of one 16-wide K sub-step: 2 weight fragments and up to 4 token fragments
+struct FragsBf16 {
+    bf16x8 a[2];
+    bf16x8 b[4];
+};
+
+template <int NTF>
+__device__ __forceinline__ void fetch_bf16(FragsBf16 &fr, const char *tok, const char *wgt, const int (&wrow)[2],
+                                           int lane, int j) {
+    const int r = lane & 31, half = lane >> 5, sx = (lane >> 1) & 7;
+    const int off = r * kRowBytes + (((2 * j + half) ^ sx) << 4);
+#pragma unroll
+    for (int f = 0; f < 2; ++f) fr.a[f] = *reinterpret_cast<const bf16x8 *>(wgt + wrow[f] * kRowBytes + off);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+        if (t < NTF) fr.b[t] = *reinterpret_cast<const bf16x8 *>(tok + t * 32 * kRowBytes + off);
+}
+
+template <int NTF, bool TRANSPOSED>
+__device__ __forceinline__ void mma_bf16(f32x16 (&acc)[2][4], const FragsBf16 &fr) {
+#pragma unroll
+    for (int f = 0; f < 2; ++f)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if (t < NTF) {
+                if constexpr (TRANSPOSED)
+                    acc[f][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.a[f], fr.b[t], acc[f][t], 0, 0, 0);
+                else
+                    acc[f][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.b[t], fr.a[f], acc[f][t], 0, 0, 0);
+            }
+}
+
+// ------------------------------------------------------------------------------------------
+// MFMA over one 128-byte slab.  `tok` points at this wave's group of 128 token rows, `wgt` at the
+// 256 weight rows of a stage.  wrow[f] = first LDS weight row of this wave's fragment f.
+// TRANSPOSED: weight rows on the MFMA M side (accumulator registers run along weight rows, lanes
+// along tokens); otherwise tokens on the M side (lanes run along weight rows).
+template <int DT, int NTF, bool TRANSPOSED, bool PREFETCH>
 __device__ __forceinline__ void mfma_slab(f32x16 (&acc)[2][4], const char *tok, const char *wgt,
                                           const int (&wrow)[2], int lane, const uint32_t (&stok)[4],
                                           const uint32_t (&sw)[2]) {
@@ -136,25 +223,37 @@ __device__ __forceinline__ void mfma_slab(f32x16 (&acc)[2][4], const char *tok, 
     const int sx = (lane >> 1) & 7;  // swz(row) for rows that are 32-aligned + r
     const int rowoff = r * kRowBytes;
     if constexpr (DT == DT_BF16) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        // PREFETCH: operand fragments are double-buffered in registers, the reads of sub-step j+1 are
+        // issued before the MFMAs of sub-step j (one wave per SIMD has nobody else to cover its LDS
+        // latency); without it one buffer is reused, which saves 24 registers.
+        bf16x8 a[2][2], b[2][4];
+        auto fetch = [&](int j, int buf) {
             const int slot = ((2 * j + half) ^ sx) << 4;
-            bf16x8 a[2], b[4];
 #pragma unroll
             for (int f = 0; f < 2; ++f)
-                a[f] = *reinterpret_cast<const bf16x8 *>(wgt + wrow[f] * kRowBytes + rowoff + slot);
+                a[buf][f] = *reinterpret_cast<const bf16x8 *>(wgt + wrow[f] * kRowBytes + rowoff + slot);
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-                if (t < NTF) b[t] = *reinterpret_cast<const bf16x8 *>(tok + t * 32 * kRowBytes + rowoff + slot);
+                if (t < NTF) b[buf][t] = *reinterpret_cast<const bf16x8 *>(tok + t * 32 * kRowBytes + rowoff + slot);
+        };
+        if constexpr (PREFETCH) fetch(0, 0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int cur = PREFETCH ? (j & 1) : 0;
+            if constexpr (PREFETCH) {
+                if (j + 1 < 4) fetch(j + 1, cur ^ 1);
+            } else {
+                fetch(j, 0);
+            }
 #pragma unroll
             for (int f = 0; f < 2; ++f)
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
                     if (t < NTF) {
                         if constexpr (TRANSPOSED)
-                            acc[f][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[f], b[t], acc[f][t], 0, 0, 0);
+                            acc[f][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cur][f], b[cur][t], acc[f][t], 0, 0, 0);
                         else
-                            acc[f][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[t], a[f], acc[f][t], 0, 0, 0);
+                            acc[f][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[cur][t], a[cur][f], acc[f][t], 0, 0, 0);
                     }
         }
     } else {
@@ -165,8 +264,10 @@ __device__ __forceinline__ void mfma_slab(f32x16 (&acc)[2][4], const char *tok, 
             // < 32 and that of block 2j+1 from lanes >= 32 (measured on gfx950).
             const int slot = ((4 * j + half) ^ sx) << 4;
             const int sh = 8 * (2 * j + half);  // the scale byte this lane supplies
-            i32x8 a[2], b[4];
-            int sa[2], sb[4];
+            // weight fragments of the sub-step stay in registers, token fragments stream through one
+            // register set (8 VGPRs) to keep the kernel within 256 registers at two waves per SIMD
+            i32x8 a[2];
+            int sa[2];
 #pragma unroll
             for (int f = 0; f < 2; ++f) {
                 const char *p = wgt + wrow[f] * kRowBytes + rowoff;
@@ -181,21 +282,19 @@ __device__ __forceinline__ void mfma_slab(f32x16 (&acc)[2][4], const char *tok, 
                     const char *p = tok + t * 32 * kRowBytes + rowoff;
                     i32x4 lo = *reinterpret_cast<const i32x4 *>(p + slot);
                     i32x4 hi = *reinterpret_cast<const i32x4 *>(p + (slot ^ 32));
-                    b[t] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-                    sb[t] = (int)((stok[t] >> sh) & 0xffu);
-                }
+                    const i32x8 b = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                    const int sb = (int)((stok[t] >> sh) & 0xffu);
 #pragma unroll
-            for (int f = 0; f < 2; ++f)
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    if (t < NTF) {
+                    for (int f = 0; f < 2; ++f) {
                         if constexpr (TRANSPOSED)
                             acc[f][t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                                a[f], b[t], acc[f][t], 0, 0, 0, sa[f], 0, sb[t]);
+                                a[f], b, acc[f][t], 0, 0, 0, sa[f], 0, sb);
                         else
                             acc[f][t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                                b[t], a[f], acc[f][t], 0, 0, 0, sb[t], 0, sa[f]);
+                                b, a[f], acc[f][t], 0, 0, 0, sb, 0, sa[f]);
                     }
+                    if constexpr (!PREFETCH) __builtin_amdgcn_sched_barrier(0);  // keep the next fragment's reads behind these MFMAs
+                }
         }
     }
 }

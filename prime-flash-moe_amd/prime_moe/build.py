@@ -21,7 +21,9 @@ SOURCES = ["api.hip", "moe_align.hip", "quantize_mx.hip", "fused_moe.hip"]
 ARCH = "gfx950"
 
 # Packed-fp32 VALU forms are switched off for every device compile.
-DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# Private arrays are never moved into LDS by the compiler: the kernels budget LDS themselves.
+DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                "-mllvm", "-disable-promote-alloca-to-lds"]
 
 
 def hipcc() -> str:

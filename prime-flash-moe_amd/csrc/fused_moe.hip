@@ -13,8 +13,8 @@
 //                -> finalize (out += bf16(accum)).
 // The top-k reduction is exact in fp32 up to summation order; `out` is rounded to bf16 once.
 #include <algorithm>
-#include <type_traits>
 
+#include "moe_ring.h"
 #include "moe_tile.h"
 #include "pmoe_common.h"
 
@@ -125,142 +125,6 @@ __device__ __forceinline__ int load_row_info(const MoeArgs &a, int first, int nb
     return m;
 }
 
-// K loop of one tile: double-buffered LDS stages, prefetch of slab k+1 while slab k computes.
-// COMPUTE = false is the loop of the waves of a group without live rows: they only take part in
-// the copies and barriers (same barrier count, no matrix work, no accumulator traffic).
-template <int DT, int NG, int NTF, bool TRANSPOSED, bool COMPUTE>
-__device__ __forceinline__ void tile_main_loop(f32x16 (&acc)[2][4], StageLoader<NG> &ld, char *lds,
-                                               int n_slabs, const int (&wrow)[2], int lane, int grp,
-                                               const uint8_t *tok_sc_base,
-                                               const uint32_t (&tok_sc)[4], const uint8_t *w_sc_base,
-                                               const uint32_t (&w_sc)[2]) {
-    using G = Geo<NG>;
-    uint32_t stok[4] = {0, 0, 0, 0}, sw[2] = {0, 0};
-    uint32_t ntok[4] = {0, 0, 0, 0}, nw[2] = {0, 0};
-    ld.load_tok(0);
-    ld.load_w(0);
-    if constexpr (DT == DT_FP8 && COMPUTE) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-            if (t < NTF) stok[t] = *reinterpret_cast<const uint32_t *>(tok_sc_base + tok_sc[t]);
-#pragma unroll
-        for (int f = 0; f < 2; ++f) sw[f] = *reinterpret_cast<const uint32_t *>(w_sc_base + w_sc[f]);
-    }
-    ld.store_tok(lds);
-    ld.store_w(lds);
-    __syncthreads();
-    for (int kt = 0; kt < n_slabs; ++kt) {
-        char *cur = lds + (kt & 1) * G::kStageBytes;
-        char *nxt = lds + ((kt + 1) & 1) * G::kStageBytes;
-        const bool more = kt + 1 < n_slabs;
-        if (more) {
-            ld.load_tok((uint32_t)(kt + 1) * kRowBytes);
-            ld.load_w((uint32_t)(kt + 1) * kRowBytes);
-            if constexpr (DT == DT_FP8 && COMPUTE) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    if (t < NTF) ntok[t] = *reinterpret_cast<const uint32_t *>(tok_sc_base + (tok_sc[t] + (uint32_t)(kt + 1) * 4));
-#pragma unroll
-                for (int f = 0; f < 2; ++f)
-                    nw[f] = *reinterpret_cast<const uint32_t *>(w_sc_base + (w_sc[f] + (uint32_t)(kt + 1) * 512));
-            }
-        }
-        if constexpr (COMPUTE)
-            mfma_slab<DT, NTF, TRANSPOSED, NG == 1>(acc, cur + grp * kGroupRegion, cur + G::kTokRegion, wrow, lane, stok, sw);
-        if (more) {
-            ld.store_tok(nxt);
-            ld.store_w(nxt);
-            if constexpr (DT == DT_FP8 && COMPUTE) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t) stok[t] = ntok[t];
-#pragma unroll
-                for (int f = 0; f < 2; ++f) sw[f] = nw[f];
-            }
-        }
-        __syncthreads();
-    }
-}
-
-// K loop of the two-group kernels: the next slab is copied global -> LDS by the DMA path while the
-// current one is consumed, one barrier per slab.  For bf16 the MFMAs are software-pipelined across
-// that barrier: the last K sub-step of a slab is held back and issued after the barrier, behind the
-// first fragment reads of the next slab, so the matrix pipe has work while LDS latency elapses.
-template <int DT, int NG, int NTF, bool TRANSPOSED, bool COMPUTE>
-__device__ __forceinline__ void tile_main_loop_dma(f32x16 (&acc)[2][4], const DmaLoader<NG> &ld, char *lds,
-                                                   int n_slabs, const int (&wrow)[2], int lane, int grp,
-                                                   const uint8_t *tok_sc_base, const uint32_t (&tok_sc)[4],
-                                                   const uint8_t *w_sc_base, const uint32_t (&w_sc)[2]) {
-    using G = Geo<NG>;
-    ld.issue(lds, 0);
-    uint32_t stok[4] = {0, 0, 0, 0}, sw[2] = {0, 0};
-    uint32_t ntok[4] = {0, 0, 0, 0}, nw[2] = {0, 0};
-    if constexpr (DT == DT_FP8 && COMPUTE) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-            if (t < NTF) stok[t] = *reinterpret_cast<const uint32_t *>(tok_sc_base + tok_sc[t]);
-#pragma unroll
-        for (int f = 0; f < 2; ++f) sw[f] = *reinterpret_cast<const uint32_t *>(w_sc_base + w_sc[f]);
-    }
-    FragsBf16 fx, fy;  // fy carries the held-back sub-step across the barrier
-    if constexpr (DT == DT_BF16 && COMPUTE) {
-#pragma unroll
-        for (int f = 0; f < 2; ++f)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) fy.a[f][i] = (__bf16)0.0f;
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) fy.b[t][i] = (__bf16)0.0f;
-    }
-    DmaLoader<NG>::wait_all();
-    __syncthreads();  // this wave's copies have landed; now everybody else's have too
-    // One slab: `cur` is read with ds_read while `nxt` is being filled by the copies issued here.
-    auto slab = [&](const char *cur, char *nxt, int kt) __attribute__((always_inline)) {
-        const bool more = kt + 1 < n_slabs;
-        if (more) {
-            ld.issue(nxt, (uint32_t)(kt + 1) * kRowBytes);
-            if constexpr (DT == DT_FP8 && COMPUTE) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    if (t < NTF) ntok[t] = *reinterpret_cast<const uint32_t *>(tok_sc_base + (tok_sc[t] + (uint32_t)(kt + 1) * 4));
-#pragma unroll
-                for (int f = 0; f < 2; ++f)
-                    nw[f] = *reinterpret_cast<const uint32_t *>(w_sc_base + (w_sc[f] + (uint32_t)(kt + 1) * 512));
-            }
-        }
-        if constexpr (COMPUTE) {
-            const char *tok = cur + grp * kGroupRegion;
-            const char *wgt = cur + G::kTokRegion;
-            if constexpr (DT == DT_BF16) {
-                fetch_bf16<NTF>(fx, tok, wgt, wrow, lane, 0);
-                mma_bf16<NTF, TRANSPOSED>(acc, fy);  // sub-step 3 of the previous slab (zeros the first time)
-                fetch_bf16<NTF>(fy, tok, wgt, wrow, lane, 1);
-                mma_bf16<NTF, TRANSPOSED>(acc, fx);
-                fetch_bf16<NTF>(fx, tok, wgt, wrow, lane, 2);
-                mma_bf16<NTF, TRANSPOSED>(acc, fy);
-                fetch_bf16<NTF>(fy, tok, wgt, wrow, lane, 3);
-                mma_bf16<NTF, TRANSPOSED>(acc, fx);
-            } else {
-                mfma_slab<DT, NTF, TRANSPOSED, false>(acc, tok, wgt, wrow, lane, stok, sw);
-#pragma unroll
-                for (int t = 0; t < 4; ++t) stok[t] = ntok[t];
-#pragma unroll
-                for (int f = 0; f < 2; ++f) sw[f] = nw[f];
-            }
-        }
-        DmaLoader<NG>::wait_all();
-        __syncthreads();
-    };
-    char *const s0 = lds, *const s1 = lds + G::kStageBytes;
-    int kt = 0;
-    for (; kt + 1 < n_slabs; kt += 2) {
-        slab(s0, s1, kt);
-        slab(s1, s0, kt + 1);
-    }
-    if (kt < n_slabs) slab(s0, s1, kt);
-    if constexpr (DT == DT_BF16 && COMPUTE) mma_bf16<NTF, TRANSPOSED>(acc, fy);
-}
-
 __device__ __forceinline__ void zero_acc(f32x16 (&acc)[2][4]) {
 #pragma unroll
     for (int f = 0; f < 2; ++f)
@@ -298,166 +162,357 @@ __device__ __forceinline__ void scatter_add(const f32x16 (&acc)[2][4], const int
     }
 }
 
-// ------------------------------------------------------------------------------------------
-// Up kernel (and, with FUSED, the whole split==0 pipeline).
-// Tile: NG row blocks x activation columns [128*ht, 128*ht+128).  LDS weight rows 0..127 are
-// gate rows, 128..255 the matching up rows; wave v of a group owns gate/up rows 32v..32v+31 so
-// gate and up of one activation element sit in the same lane and register.  Weight rows go on
-// the MFMA M side: a lane then holds 16 of the 32 activation columns of one MX block of its
-// token and the block maximum needs a single cross-lane exchange.
-template <int DT, bool FUSED, int NG, int NTF>
-__device__ __forceinline__ void up_tile(const MoeArgs &a, int first, int nb, int ht, int e,
-                                        RowInfo<NG> &ri, char *lds, char *act_lds, uint32_t *act_sc_lds) {
-    using G = Geo<NG>;
-    constexpr int ES = DT == DT_BF16 ? 2 : 1;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
+// SwiGLU epilogue of the up GEMM, in registers: the 2H-wide gate/up tensor never leaves the chip.
+// acc[0] holds gate rows, acc[1] the matching up rows (weight rows on the MFMA M side: register i
+// of lane l = activation column 32 w4 + 8(i/4) + 4(l/32) + i%4 of token row 32 t + l%32).  The
+// 128 x 128 activation tile of the group is written to `tile`:
+//   OPERAND = false: row pitch kActPitch*, for the coalesced copy to the workspace;
+//   OPERAND = true : in the 128-byte-slab MFMA operand layout of the fused kernel's down phase.
+// mxfp8: per token row and 32 columns, amax -> e8m0 scale + e4m3 values; a lane holds 16 of the 32
+// columns of one MX block, the partner lane (l ^ 32) the others.
+template <int DT, bool OPERAND, int NTF>
+__device__ __forceinline__ void swiglu_epilogue(const f32x16 (&acc)[2][4], char *tile, uint32_t *sc_tile,
+                                                int w4, int lane) {
     const int r = lane & 31, half = lane >> 5;
-    const int K = a.K, H = a.H, N = a.N;
-    const int h0 = ht * 128;
-    const int my_ntf = (ri.nvalid[grp] + 31) >> 5;
-    const bool active = __builtin_amdgcn_readfirstlane(my_ntf) > 0;
-
-    // NG == 2: DMA copies (the lane landing in LDS slot `chunk` fetches global chunk chunk ^ swz);
-    // NG == 1: register-staged copies (the thread fetching global chunk `chunk` writes slot chunk ^ swz)
-    typename std::conditional<NG == 2, DmaLoader<NG>, StageLoader<NG>>::type ld;
-    const int lrow = tid >> 3, chunk = tid & 7;
-    const int gchunk = NG == 2 ? (chunk ^ swz(lrow)) : chunk;
-    if constexpr (NG == 2) ld.lds_wave_off = __builtin_amdgcn_readfirstlane((tid >> 6) * 8 * kRowBytes);
-    else ld.lds_off = lrow * kRowBytes + ((chunk ^ swz(lrow)) << 4);
-    ld.tok_mask = 0;
 #pragma unroll
-    for (int i = 0; i < G::kTokPasses; ++i) {
-        const int row = lrow + i * G::kPassRows;
-        int tok = ri.tok[row];
-        if (tok < 0) tok = 0;
-        ld.tok_off[i] = (uint32_t)tok * (uint32_t)(K * ES) + gchunk * 16;
-        if (((row & 127) >> 5) < ((ri.nvalid[row >> 7] + 31) >> 5)) ld.tok_mask |= 1 << i;
-    }
-    ld.tok_mask = __builtin_amdgcn_readfirstlane(ld.tok_mask);  // a wave's 8 rows share a fragment
-    ld.tok_base = a.x;
-    ld.w_base[0] = a.w1 + ((int64_t)e * N + h0) * K * ES;
-    ld.w_base[1] = ld.w_base[0] + (int64_t)H * K * ES;
-    ld.w_off = (uint32_t)lrow * (uint32_t)(K * ES) + gchunk * 16;
-    ld.w_pitch_pass = (uint32_t)G::kPassRows * (uint32_t)(K * ES);
-
-    const int wrow[2] = {32 * w4, 128 + 32 * w4};
-    uint32_t tok_sc[4] = {0, 0, 0, 0}, w_sc[2] = {0, 0};
-    const uint8_t *tok_sc_base = a.x_scales, *w_sc_base = nullptr;
-    if constexpr (DT == DT_FP8) {
-        const int kb = K >> 5;
+    for (int t = 0; t < 4; ++t) {
+        if (t < NTF) {
+            float v[16];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            int tok = ri.tok[grp * kBlockRows + 32 * t + r];
-            if (tok < 0) tok = 0;
-            tok_sc[t] = (uint32_t)tok * (uint32_t)kb;
-        }
-        w_sc_base = a.w1_scales + (int64_t)e * N * kb;
-        w_sc[0] = (uint32_t)blocked_scale_off(h0 + 32 * w4 + r, 0, K >> 7);
-        w_sc[1] = (uint32_t)blocked_scale_off(H + h0 + 32 * w4 + r, 0, K >> 7);
-    }
-
-    f32x16 acc[2][4];
-    zero_acc(acc);
-    if constexpr (NG == 2) {
-        if (active)
-            tile_main_loop_dma<DT, NG, NTF, true, true>(acc, ld, lds, (K * ES) / kRowBytes, wrow, lane, grp,
-                                                        tok_sc_base, tok_sc, w_sc_base, w_sc);
-        else
-            tile_main_loop_dma<DT, NG, NTF, true, false>(acc, ld, lds, (K * ES) / kRowBytes, wrow, lane, grp,
-                                                         tok_sc_base, tok_sc, w_sc_base, w_sc);
-    } else {
-        tile_main_loop<DT, NG, NTF, true, true>(acc, ld, lds, (K * ES) / kRowBytes, wrow, lane, grp, tok_sc_base,
-                                                tok_sc, w_sc_base, w_sc);
-    }
-
-    // ---- epilogue: SwiGLU in registers; the 2H-wide gate/up tensor never leaves the chip ----
-    // (the main loop ended with a barrier, so the stage buffers may be overwritten)
-    constexpr int kPitch = DT == DT_BF16 ? kActPitchBf16 : kActPitchFp8;
-    char *tile = FUSED ? act_lds : lds + grp * (kBlockRows * kPitch);
-    uint32_t *sc_tile = act_sc_lds + grp * kBlockRows;
-    if (active) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            if (t < NTF) {
-                float v[16];
-#pragma unroll
-                for (int i = 0; i < 16; ++i) v[i] = swiglu(acc[0][t][i], acc[1][t][i]);
-                const int row = 32 * t + r;
-                if constexpr (DT == DT_BF16) {
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const int hl = 32 * w4 + 8 * g + 4 * half;  // tile-local activation column
-                        uint2 pk;
-                        pk.x = f32_to_bf16_bits(v[4 * g]) | (f32_to_bf16_bits(v[4 * g + 1]) << 16);
-                        pk.y = f32_to_bf16_bits(v[4 * g + 2]) | (f32_to_bf16_bits(v[4 * g + 3]) << 16);
-                        char *dst;
-                        if constexpr (FUSED) {
-                            const int byte = (hl & 63) * 2;
-                            dst = tile + (hl >> 6) * kGroupRegion + row * kRowBytes +
-                                  (((byte >> 4) ^ swz(row)) << 4) + (byte & 15);
-                        } else {
-                            dst = tile + row * kActPitchBf16 + hl * 2;
-                        }
-                        *reinterpret_cast<uint2 *>(dst) = pk;
-                    }
-                } else {
-                    float amax = 0.f;
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(v[i]));
-                    amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-                    uint32_t e8;
-                    float inv;
-                    mx_block_scale(amax, e8, inv);
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const int hl = 32 * w4 + 8 * g + 4 * half;
-                        const uint32_t q = pack4_e4m3(v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3], inv);
-                        char *dst;
-                        if constexpr (FUSED)
-                            dst = tile + row * kRowBytes + (((hl >> 4) ^ swz(row)) << 4) + (hl & 15);
-                        else
-                            dst = tile + row * kActPitchFp8 + hl;
-                        *reinterpret_cast<uint32_t *>(dst) = q;
-                    }
-                    if (half == 0) reinterpret_cast<uint8_t *>(sc_tile)[row * 4 + w4] = (uint8_t)e8;
-                }
-            }
-        }
-    }
-    __syncthreads();
-    if constexpr (!FUSED) {
-        // coalesced copy of the live rows of the group's tile to the activation workspace
-        if (active) {
-            const int64_t row0 = (int64_t)(first + grp) * kBlockRows;
+            for (int i = 0; i < 16; ++i) v[i] = swiglu(acc[0][t][i], acc[1][t][i]);
+            const int row = 32 * t + r;
             if constexpr (DT == DT_BF16) {
-                const int c = gt & 15;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int row = (gt >> 4) + 16 * i;
-                    if (row < 32 * my_ntf) {
-                        uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchBf16 + c * 16);
-                        *reinterpret_cast<uint4 *>(a.act + ((row0 + row) * H + h0) * 2 + c * 16) = v;
+                for (int g = 0; g < 4; ++g) {
+                    const int hl = 32 * w4 + 8 * g + 4 * half;  // tile-local activation column
+                    uint2 pk;
+                    pk.x = f32_to_bf16_bits(v[4 * g]) | (f32_to_bf16_bits(v[4 * g + 1]) << 16);
+                    pk.y = f32_to_bf16_bits(v[4 * g + 2]) | (f32_to_bf16_bits(v[4 * g + 3]) << 16);
+                    char *dst;
+                    if constexpr (OPERAND) {
+                        const int byte = (hl & 63) * 2;
+                        dst = tile + (hl >> 6) * kGroupRegion + row * kRowBytes +
+                              (((byte >> 4) ^ swz(row)) << 4) + (byte & 15);
+                    } else {
+                        dst = tile + row * kActPitchBf16 + hl * 2;
                     }
+                    *reinterpret_cast<uint2 *>(dst) = pk;
                 }
             } else {
-                const int c = gt & 7;
+                float amax = 0.f;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int row = (gt >> 3) + 32 * i;
-                    if (i < my_ntf) {
-                        uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchFp8 + c * 16);
-                        *reinterpret_cast<uint4 *>(a.act + (row0 + row) * H + h0 + c * 16) = v;
-                    }
+                for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(v[i]));
+                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+                uint32_t e8;
+                float inv;
+                mx_block_scale(amax, e8, inv);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int hl = 32 * w4 + 8 * g + 4 * half;
+                    const uint32_t q = pack4_e4m3(v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3], inv);
+                    char *dst;
+                    if constexpr (OPERAND)
+                        dst = tile + row * kRowBytes + (((hl >> 4) ^ swz(row)) << 4) + (hl & 15);
+                    else
+                        dst = tile + row * kActPitchFp8 + hl;
+                    *reinterpret_cast<uint32_t *>(dst) = q;
                 }
-                if (gt < 32 * my_ntf)
-                    *reinterpret_cast<uint32_t *>(a.act_scales + (row0 + gt) * (H >> 5) + ht * 4) = sc_tile[gt];
+                if (half == 0) reinterpret_cast<uint8_t *>(sc_tile)[row * 4 + w4] = (uint8_t)e8;
             }
         }
     }
 }
 
-// Down phase of the split==0 pipeline: the activation tile (128 rows x 128 columns of H) stays in
+// Coalesced copy of the first 32*ntf rows of a group's activation tile (pitch kActPitch*) to the
+// workspace rows row0.., columns [h0, h0+128); gt = thread index inside the group (0..255).
+template <int DT>
+__device__ __forceinline__ void store_act_tile(const MoeArgs &a, const char *tile, const uint32_t *sc_tile,
+                                               int64_t row0, int h0, int ntf, int gt) {
+    const int H = a.H;
+    if constexpr (DT == DT_BF16) {
+        const int c = gt & 15;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int row = (gt >> 4) + 16 * i;
+            if (row < 32 * ntf) {
+                uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchBf16 + c * 16);
+                *reinterpret_cast<uint4 *>(a.act + ((row0 + row) * H + h0) * 2 + c * 16) = v;
+            }
+        }
+    } else {
+        const int c = gt & 7;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = (gt >> 3) + 32 * i;
+            if (i < ntf) {
+                uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchFp8 + c * 16);
+                *reinterpret_cast<uint4 *>(a.act + (row0 + row) * H + h0 + c * 16) = v;
+            }
+        }
+        if (gt < 32 * ntf)
+            *reinterpret_cast<uint32_t *>(a.act_scales + (row0 + gt) * (H >> 5) + (h0 >> 7) * 4) = sc_tile[gt];
+    }
+}
+
+// ==========================================================================================
+// Split pipeline, two-group kernels on the ring engine
+// ==========================================================================================
+
+// Common set-up of the ring loader.  Token rows: `tok_row_off(row)` gives the byte offset of tile
+// row `row` (0..255) in `tok_base`; weight rows: the tile's two 128-row halves start at w_base[0/1]
+// with `w_pitch` bytes per row.  Scales (mxfp8): `tok_sc_off(row)` / `w_sc_off(row)` are the byte
+// offsets of the row's first 4-scale dword.
+template <int DT, typename TokOff, typename TokScOff, typename WScOff>
+__device__ __forceinline__ void setup_ring_loader(ring::Loader &ld, int tid, uint32_t w_pitch, TokOff tok_row_off,
+                                                  const uint8_t *tok_sc_base, TokScOff tok_sc_off,
+                                                  const uint8_t *w_sc_base, WScOff w_sc_off) {
+    const int wave = tid >> 6, lane = tid & 63;
+    const int prow = tid >> 2;                      // row inside a 128-row pass
+    const int gchunk = (tid & 3) ^ ring::swz64(prow);  // global chunk landing in this lane's LDS slot
+    ld.tok_off[0] = tok_row_off(prow) + gchunk * 16;
+    ld.tok_off[1] = tok_row_off(kBlockRows + prow) + gchunk * 16;
+    ld.w_off = (uint32_t)prow * w_pitch + gchunk * 16;
+    ld.wave_off = __builtin_amdgcn_readfirstlane(wave * 16 * ring::kRB);
+    ld.wave_sc_off = __builtin_amdgcn_readfirstlane(wave * 64 * 4);
+    ld.sc_base = nullptr;
+    ld.sc_off = 0;
+    ld.sc_step = 0;
+    if constexpr (DT == DT_FP8) {
+        const int row = wave * 64 + lane;  // 0..255 token rows, 256..511 weight rows
+        const bool is_tok = __builtin_amdgcn_readfirstlane(wave) < 4;
+        ld.sc_base = reinterpret_cast<const char *>(is_tok ? tok_sc_base : w_sc_base);
+        ld.sc_off = is_tok ? tok_sc_off(row) : w_sc_off(row - ring::kTokRows);
+        ld.sc_step = is_tok ? 4u : 512u;
+    }
+}
+
+// First slab of this workgroup's walk over K: workgroups that run side by side on an XCD (consecutive
+// blockIdx / 8) start 256 bytes apart, 16 distinct phases over a 4 KB period.
+__device__ __forceinline__ int slab_rotation(int n_slabs) {
+    const int phase = (int)((blockIdx.x >> 3) & 15) * (256 / ring::kRB);
+    return phase % n_slabs & ~1;
+}
+
+// Up kernel tile: NG = 2 row blocks x activation columns [128 ht, 128 ht + 128).  LDS weight rows
+// 0..127 are gate rows, 128..255 the matching up rows; wave v of a group owns gate/up rows
+// 32v..32v+31 so gate and up of one activation element sit in the same lane and register.
+template <int DT, int NTF>
+__device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht, int e, RowInfo<2> &ri,
+                                             char *lds, uint32_t *act_sc_lds) {
+    constexpr int ES = DT == DT_BF16 ? 2 : 1;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
+    const int K = a.K, H = a.H, N = a.N;
+    const int h0 = ht * 128;
+    const int my_ntf = __builtin_amdgcn_readfirstlane((ri.nvalid[grp] + 31) >> 5);
+    const bool active = my_ntf > 0;
+
+    ring::Loader ld;
+    ld.tok_base = a.x;
+    ld.w_base[0] = a.w1 + ((int64_t)e * N + h0) * K * ES;
+    ld.w_base[1] = ld.w_base[0] + (int64_t)H * K * ES;
+    const uint32_t row_bytes = (uint32_t)(K * ES);
+    const int kb = K >> 5;
+    setup_ring_loader<DT>(
+        ld, tid, row_bytes,
+        [&](int row) { return (uint32_t)max(ri.tok[row], 0) * row_bytes; },  // dead rows read token 0
+        a.x_scales, [&](int row) { return (uint32_t)max(ri.tok[row], 0) * (uint32_t)kb; },
+        a.w1_scales + (int64_t)e * N * kb,
+        [&](int row) { return (uint32_t)blocked_scale_off((row < 128 ? h0 : H + h0 - 128) + row, 0, K >> 7); });
+
+    const int wrow[2] = {32 * w4, 128 + 32 * w4};
+    f32x16 acc[2][4];
+    zero_acc(acc);
+    const int n_slabs = (K * ES) / ring::kRB;
+    const int start = slab_rotation(n_slabs);
+    if (active) ring::main_loop<DT, NTF, true, true>(acc, ld, lds, n_slabs, wrow, lane, grp, start);
+    else ring::main_loop<DT, NTF, true, false>(acc, ld, lds, n_slabs, wrow, lane, grp, start);
+
+    // the ring is free (main_loop ends with a barrier): reuse it for the activation tiles
+    constexpr int kPitch = DT == DT_BF16 ? kActPitchBf16 : kActPitchFp8;
+    char *tile = lds + grp * (kBlockRows * kPitch);
+    uint32_t *sc_tile = act_sc_lds + grp * kBlockRows;
+    if (active) swiglu_epilogue<DT, false, NTF>(acc, tile, sc_tile, w4, lane);
+    __syncthreads();
+    if (active) store_act_tile<DT>(a, tile, sc_tile, (int64_t)(first + grp) * kBlockRows, h0, my_ntf, gt);
+}
+
+template <int DT>
+__global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
+    __shared__ __attribute__((aligned(1024))) char lds[ring::kStages * ring::stage_bytes<DT>()];
+    __shared__ uint32_t act_sc_lds[kBlockRows * 2];
+    __shared__ RowInfo<2> ri;
+    int first, nb, ht;
+    if (!resolve_tile<2>(a, first, nb, ht)) return;
+    if (first * kBlockRows >= a.ntpp[0]) return;
+    const int ntf = load_row_info<2>(a, first, nb, ri);
+    if (ntf == 0) return;
+    const int e = a.expert_ids[first];
+    if (e < 0 || e >= a.E) return;
+    if (ntf == 1) up_tile_ring<DT, 1>(a, first, ht, e, ri, lds, act_sc_lds);
+    else if (ntf == 2) up_tile_ring<DT, 2>(a, first, ht, e, ri, lds, act_sc_lds);
+    else up_tile_ring<DT, 4>(a, first, ht, e, ri, lds, act_sc_lds);
+}
+
+// Down kernel of the split pipeline: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
+// full reduction over H inside the workgroup (no split-K), then w[row] * y added to accum[token].
+template <int DT, int NTF>
+__device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, char *lds) {
+    constexpr int ES = DT == DT_BF16 ? 2 : 1;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int grp = wave >> 2, w4 = wave & 3;
+    const int K = a.K, H = a.H;
+    const int k0 = kt * kWRows;
+    const int64_t row0 = (int64_t)first * kBlockRows;
+    const bool active = __builtin_amdgcn_readfirstlane(ri.nvalid[grp]) > 0;
+
+    ring::Loader ld;
+    ld.tok_base = a.act + row0 * H * ES;
+    ld.w_base[0] = a.w2 + ((int64_t)e * K + k0) * H * ES;
+    ld.w_base[1] = (k0 + 128 < K) ? ld.w_base[0] + (int64_t)128 * H * ES : ld.w_base[0];
+    const uint32_t row_bytes = (uint32_t)(H * ES);
+    const int hb = H >> 5;
+    // rows of a block that does not belong to this tile (single tiles) re-read the tile's row 0
+    const int live_rows = __builtin_amdgcn_readfirstlane(ri.nvalid[1] > 0 ? 2 * kBlockRows : kBlockRows);
+    setup_ring_loader<DT>(
+        ld, tid, row_bytes, [&](int row) { return (uint32_t)(row < live_rows ? row : 0) * row_bytes; },
+        a.act_scales + row0 * hb, [&](int row) { return (uint32_t)(row < live_rows ? row : 0) * (uint32_t)hb; },
+        a.w2_scales + (int64_t)e * K * hb,
+        [&](int row) { return (uint32_t)blocked_scale_off(min(k0 + row, K - 1), 0, H >> 7); });
+
+    const int wrow[2] = {64 * w4, 64 * w4 + 32};
+    f32x16 acc[2][4];
+    zero_acc(acc);
+    const int n_slabs = (H * ES) / ring::kRB;
+    const int start = slab_rotation(n_slabs);
+    if (active) {
+        ring::main_loop<DT, NTF, false, true>(acc, ld, lds, n_slabs, wrow, lane, grp, start);
+        scatter_add<NTF>(acc, ri.tok + grp * kBlockRows, ri.wt + grp * kBlockRows, a.accum, K, k0 + 64 * w4, lane);
+    } else {
+        ring::main_loop<DT, NTF, false, false>(acc, ld, lds, n_slabs, wrow, lane, grp, start);
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
+    __shared__ __attribute__((aligned(1024))) char lds[ring::kStages * ring::stage_bytes<DT>()];
+    __shared__ RowInfo<2> ri;
+    int first, nb, kt;
+    if (!resolve_tile<2>(a, first, nb, kt)) return;
+    if (first * kBlockRows >= a.ntpp[0]) return;
+    const int ntf = load_row_info<2>(a, first, nb, ri);
+    if (ntf == 0) return;
+    const int e = a.expert_ids[first];
+    if (e < 0 || e >= a.E) return;
+    if (ntf == 1) down_tile_ring<DT, 1>(a, first, kt, e, ri, lds);
+    else if (ntf == 2) down_tile_ring<DT, 2>(a, first, kt, e, ri, lds);
+    else down_tile_ring<DT, 4>(a, first, kt, e, ri, lds);
+}
+
+// ==========================================================================================
+// Fused pipeline (split == 0): one row block per 256-thread workgroup, register-staged engine
+// ==========================================================================================
+
+// K loop of one tile: double-buffered LDS stages, prefetch of slab k+1 while slab k computes.
+template <int DT, int NTF, bool TRANSPOSED>
+__device__ __forceinline__ void tile_main_loop(f32x16 (&acc)[2][4], StageLoader<1> &ld, char *lds,
+                                               int n_slabs, const int (&wrow)[2], int lane,
+                                               const uint8_t *tok_sc_base, const uint32_t (&tok_sc)[4],
+                                               const uint8_t *w_sc_base, const uint32_t (&w_sc)[2]) {
+    using G = Geo<1>;
+    uint32_t stok[4] = {0, 0, 0, 0}, sw[2] = {0, 0};
+    uint32_t ntok[4] = {0, 0, 0, 0}, nw[2] = {0, 0};
+    ld.load_tok(0);
+    ld.load_w(0);
+    if constexpr (DT == DT_FP8) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            if (t < NTF) stok[t] = *reinterpret_cast<const uint32_t *>(tok_sc_base + tok_sc[t]);
+#pragma unroll
+        for (int f = 0; f < 2; ++f) sw[f] = *reinterpret_cast<const uint32_t *>(w_sc_base + w_sc[f]);
+    }
+    ld.store_tok(lds);
+    ld.store_w(lds);
+    __syncthreads();
+    for (int kt = 0; kt < n_slabs; ++kt) {
+        char *cur = lds + (kt & 1) * G::kStageBytes;
+        char *nxt = lds + ((kt + 1) & 1) * G::kStageBytes;
+        const bool more = kt + 1 < n_slabs;
+        if (more) {
+            ld.load_tok((uint32_t)(kt + 1) * kRowBytes);
+            ld.load_w((uint32_t)(kt + 1) * kRowBytes);
+            if constexpr (DT == DT_FP8) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (t < NTF) ntok[t] = *reinterpret_cast<const uint32_t *>(tok_sc_base + (tok_sc[t] + (uint32_t)(kt + 1) * 4));
+#pragma unroll
+                for (int f = 0; f < 2; ++f)
+                    nw[f] = *reinterpret_cast<const uint32_t *>(w_sc_base + (w_sc[f] + (uint32_t)(kt + 1) * 512));
+            }
+        }
+        mfma_slab<DT, NTF, TRANSPOSED, true>(acc, cur, cur + G::kTokRegion, wrow, lane, stok, sw);
+        if (more) {
+            ld.store_tok(nxt);
+            ld.store_w(nxt);
+            if constexpr (DT == DT_FP8) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) stok[t] = ntok[t];
+#pragma unroll
+                for (int f = 0; f < 2; ++f) sw[f] = nw[f];
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// Up phase of the fused kernel: leaves the SwiGLU (and, for mxfp8, requantised) 128 x 128
+// activation tile in LDS in MFMA operand layout.
+template <int DT, int NTF>
+__device__ __forceinline__ void fused_up_phase(const MoeArgs &a, int ht, int e, RowInfo<1> &ri, char *lds,
+                                               char *act_lds, uint32_t *act_sc_lds) {
+    using G = Geo<1>;
+    constexpr int ES = DT == DT_BF16 ? 2 : 1;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31;
+    const int K = a.K, H = a.H, N = a.N;
+    const int h0 = ht * 128;
+
+    StageLoader<1> ld;
+    const int lrow = tid >> 3, chunk = tid & 7;
+    ld.lds_off = lrow * kRowBytes + ((chunk ^ swz(lrow)) << 4);
+    ld.tok_mask = 0;
+#pragma unroll
+    for (int i = 0; i < G::kTokPasses; ++i) {
+        const int row = lrow + i * G::kPassRows;
+        ld.tok_off[i] = (uint32_t)max(ri.tok[row], 0) * (uint32_t)(K * ES) + chunk * 16;
+        if ((row >> 5) < ((ri.nvalid[0] + 31) >> 5)) ld.tok_mask |= 1 << i;
+    }
+    ld.tok_mask = __builtin_amdgcn_readfirstlane(ld.tok_mask);  // a wave's 8 rows share a fragment
+    ld.tok_base = a.x;
+    ld.w_base[0] = a.w1 + ((int64_t)e * N + h0) * K * ES;
+    ld.w_base[1] = ld.w_base[0] + (int64_t)H * K * ES;
+    ld.w_off = (uint32_t)lrow * (uint32_t)(K * ES) + chunk * 16;
+    ld.w_pitch_pass = (uint32_t)G::kPassRows * (uint32_t)(K * ES);
+
+    const int wrow[2] = {32 * wave, 128 + 32 * wave};
+    uint32_t tok_sc[4] = {0, 0, 0, 0}, w_sc[2] = {0, 0};
+    const uint8_t *w_sc_base = nullptr;
+    if constexpr (DT == DT_FP8) {
+        const int kb = K >> 5;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) tok_sc[t] = (uint32_t)max(ri.tok[32 * t + r], 0) * (uint32_t)kb;
+        w_sc_base = a.w1_scales + (int64_t)e * N * kb;
+        w_sc[0] = (uint32_t)blocked_scale_off(h0 + 32 * wave + r, 0, K >> 7);
+        w_sc[1] = (uint32_t)blocked_scale_off(H + h0 + 32 * wave + r, 0, K >> 7);
+    }
+    f32x16 acc[2][4];
+    zero_acc(acc);
+    tile_main_loop<DT, NTF, true>(acc, ld, lds, (K * ES) / kRowBytes, wrow, lane, a.x_scales, tok_sc, w_sc_base, w_sc);
+    swiglu_epilogue<DT, true, NTF>(acc, act_lds, act_sc_lds, wave, lane);
+    __syncthreads();
+}
+
+// Down phase of the fused kernel: the activation tile (128 rows x 128 columns of H) stays in
 // LDS as the token operand; W2[e][256-row chunk][h-slice] streams through the weight region.
 template <int DT, int NTF>
 __device__ __forceinline__ void fused_down_phase(const MoeArgs &a, int ht, int e, RowInfo<1> &ri,
@@ -530,111 +585,29 @@ __device__ __forceinline__ void fused_down_phase(const MoeArgs &a, int ht, int e
     }
 }
 
-template <int DT, bool FUSED, int NG>
-__global__ __launch_bounds__(256 * NG) void moe_up_kernel(MoeArgs a) {
-    static_assert(!FUSED || NG == 1, "the fused pipeline keeps one row block per workgroup");
-    __shared__ __attribute__((aligned(1024))) char lds[kNumStages * Geo<NG>::kStageBytes];
-    __shared__ __attribute__((aligned(1024))) char act_lds[FUSED ? (DT == DT_BF16 ? 2 : 1) * kGroupRegion : 16];
-    __shared__ uint32_t act_sc_lds[kBlockRows * NG];
-    __shared__ RowInfo<NG> ri;
+template <int DT>
+__global__ __launch_bounds__(256) void moe_fused_kernel(MoeArgs a) {
+    __shared__ __attribute__((aligned(1024))) char lds[kNumStages * Geo<1>::kStageBytes];
+    __shared__ __attribute__((aligned(1024))) char act_lds[(DT == DT_BF16 ? 2 : 1) * kGroupRegion];
+    __shared__ uint32_t act_sc_lds[kBlockRows];
+    __shared__ RowInfo<1> ri;
     int first, nb, ht;
-    if (!resolve_tile<NG>(a, first, nb, ht)) return;
+    if (!resolve_tile<1>(a, first, nb, ht)) return;
     if (first * kBlockRows >= a.ntpp[0]) return;
-    const int ntf = load_row_info<NG>(a, first, nb, ri);
+    const int ntf = load_row_info<1>(a, first, nb, ri);
     if (ntf == 0) return;
     const int e = a.expert_ids[first];
     if (e < 0 || e >= a.E) return;
     if (ntf == 1) {
-        up_tile<DT, FUSED, NG, 1>(a, first, nb, ht, e, ri, lds, act_lds, act_sc_lds);
-        if constexpr (FUSED) fused_down_phase<DT, 1>(a, ht, e, ri, lds, act_lds, act_sc_lds);
+        fused_up_phase<DT, 1>(a, ht, e, ri, lds, act_lds, act_sc_lds);
+        fused_down_phase<DT, 1>(a, ht, e, ri, lds, act_lds, act_sc_lds);
     } else if (ntf == 2) {
-        up_tile<DT, FUSED, NG, 2>(a, first, nb, ht, e, ri, lds, act_lds, act_sc_lds);
-        if constexpr (FUSED) fused_down_phase<DT, 2>(a, ht, e, ri, lds, act_lds, act_sc_lds);
+        fused_up_phase<DT, 2>(a, ht, e, ri, lds, act_lds, act_sc_lds);
+        fused_down_phase<DT, 2>(a, ht, e, ri, lds, act_lds, act_sc_lds);
     } else {
-        up_tile<DT, FUSED, NG, 4>(a, first, nb, ht, e, ri, lds, act_lds, act_sc_lds);
-        if constexpr (FUSED) fused_down_phase<DT, 4>(a, ht, e, ri, lds, act_lds, act_sc_lds);
+        fused_up_phase<DT, 4>(a, ht, e, ri, lds, act_lds, act_sc_lds);
+        fused_down_phase<DT, 4>(a, ht, e, ri, lds, act_lds, act_sc_lds);
     }
-}
-
-// Down kernel of the split pipeline: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
-// full reduction over H inside the workgroup (no split-K), then w[row] * y added to accum[token].
-template <int DT, int NG, int NTF>
-__device__ __forceinline__ void down_tile(const MoeArgs &a, int first, int kt, int e, RowInfo<NG> &ri, char *lds) {
-    using G = Geo<NG>;
-    constexpr int ES = DT == DT_BF16 ? 2 : 1;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int grp = wave >> 2, w4 = wave & 3;
-    const int r = lane & 31;
-    const int K = a.K, H = a.H;
-    const int k0 = kt * kWRows;
-    const int64_t row0 = (int64_t)first * kBlockRows;
-    const bool active = __builtin_amdgcn_readfirstlane(ri.nvalid[grp]) > 0;
-
-    typename std::conditional<NG == 2, DmaLoader<NG>, StageLoader<NG>>::type ld;
-    const int lrow = tid >> 3, chunk = tid & 7;
-    const int gchunk = NG == 2 ? (chunk ^ swz(lrow)) : chunk;
-    if constexpr (NG == 2) ld.lds_wave_off = __builtin_amdgcn_readfirstlane((tid >> 6) * 8 * kRowBytes);
-    else ld.lds_off = lrow * kRowBytes + ((chunk ^ swz(lrow)) << 4);
-    ld.tok_mask = 0;
-#pragma unroll
-    for (int i = 0; i < G::kTokPasses; ++i) {
-        const int row = lrow + i * G::kPassRows;
-        ld.tok_off[i] = (uint32_t)row * (uint32_t)(H * ES) + gchunk * 16;
-        if (((row & 127) >> 5) < ((ri.nvalid[row >> 7] + 31) >> 5)) ld.tok_mask |= 1 << i;
-    }
-    ld.tok_mask = __builtin_amdgcn_readfirstlane(ld.tok_mask);  // a wave's 8 rows share a fragment
-    ld.tok_base = a.act + row0 * H * ES;
-    ld.w_base[0] = a.w2 + ((int64_t)e * K + k0) * H * ES;
-    ld.w_base[1] = (k0 + 128 < K) ? ld.w_base[0] + (int64_t)128 * H * ES : ld.w_base[0];
-    ld.w_off = (uint32_t)lrow * (uint32_t)(H * ES) + gchunk * 16;
-    ld.w_pitch_pass = (uint32_t)G::kPassRows * (uint32_t)(H * ES);
-
-    const int wrow[2] = {64 * w4, 64 * w4 + 32};
-    uint32_t tok_sc[4] = {0, 0, 0, 0}, w_sc[2] = {0, 0};
-    const uint8_t *tok_sc_base = nullptr, *w_sc_base = nullptr;
-    if constexpr (DT == DT_FP8) {
-        tok_sc_base = a.act_scales + row0 * (H >> 5);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) tok_sc[t] = (uint32_t)(grp * kBlockRows + 32 * t + r) * (uint32_t)(H >> 5);
-        w_sc_base = a.w2_scales + (int64_t)e * K * (H >> 5);
-#pragma unroll
-        for (int f = 0; f < 2; ++f) {
-            int row = k0 + 64 * w4 + 32 * f + r;
-            if (row >= K) row = K - 1;
-            w_sc[f] = (uint32_t)blocked_scale_off(row, 0, H >> 7);
-        }
-    }
-    f32x16 acc[2][4];
-    zero_acc(acc);
-    if constexpr (NG == 2) {
-        if (active)
-            tile_main_loop_dma<DT, NG, NTF, false, true>(acc, ld, lds, (H * ES) / kRowBytes, wrow, lane, grp,
-                                                         tok_sc_base, tok_sc, w_sc_base, w_sc);
-        else
-            tile_main_loop_dma<DT, NG, NTF, false, false>(acc, ld, lds, (H * ES) / kRowBytes, wrow, lane, grp,
-                                                          tok_sc_base, tok_sc, w_sc_base, w_sc);
-    } else {
-        tile_main_loop<DT, NG, NTF, false, true>(acc, ld, lds, (H * ES) / kRowBytes, wrow, lane, grp, tok_sc_base,
-                                                 tok_sc, w_sc_base, w_sc);
-    }
-    if (active)
-        scatter_add<NTF>(acc, ri.tok + grp * kBlockRows, ri.wt + grp * kBlockRows, a.accum, K, k0 + 64 * w4, lane);
-}
-
-template <int DT, int NG>
-__global__ __launch_bounds__(256 * NG) void moe_down_kernel(MoeArgs a) {
-    __shared__ __attribute__((aligned(1024))) char lds[kNumStages * Geo<NG>::kStageBytes];
-    __shared__ RowInfo<NG> ri;
-    int first, nb, kt;
-    if (!resolve_tile<NG>(a, first, nb, kt)) return;
-    if (first * kBlockRows >= a.ntpp[0]) return;
-    const int ntf = load_row_info<NG>(a, first, nb, ri);
-    if (ntf == 0) return;
-    const int e = a.expert_ids[first];
-    if (e < 0 || e >= a.E) return;
-    if (ntf == 1) down_tile<DT, NG, 1>(a, first, kt, e, ri, lds);
-    else if (ntf == 2) down_tile<DT, NG, 2>(a, first, kt, e, ri, lds);
-    else down_tile<DT, NG, 4>(a, first, kt, e, ri, lds);
 }
 
 // Prologue of every call: clears the fp32 accumulator and (workgroup 0) builds the list of row
@@ -767,13 +740,13 @@ static int launch_pipeline(MoeArgs a, void *out, int split, hipStream_t s) {
         const int grid = grid_for(a.n_blocks * a.n_wtiles);
         if (split) {
             if (mask & PMOE_PHASE_UP)
-                hipLaunchKernelGGL((moe_up_kernel<DT, false, 2>), dim3(grid), dim3(512), 0, s, a);
+                hipLaunchKernelGGL((moe_up_kernel<DT>), dim3(grid), dim3(512), 0, s, a);
             MoeArgs d = a;
             d.n_wtiles = (a.K + kWRows - 1) / kWRows;
             if (mask & PMOE_PHASE_DOWN)
-                hipLaunchKernelGGL((moe_down_kernel<DT, 2>), dim3(grid_for(d.n_blocks * d.n_wtiles)), dim3(512), 0, s, d);
+                hipLaunchKernelGGL((moe_down_kernel<DT>), dim3(grid_for(d.n_blocks * d.n_wtiles)), dim3(512), 0, s, d);
         } else if (mask & PMOE_PHASE_UP) {
-            hipLaunchKernelGGL((moe_up_kernel<DT, true, 1>), dim3(grid), dim3(256), 0, s, a);
+            hipLaunchKernelGGL((moe_fused_kernel<DT>), dim3(grid), dim3(256), 0, s, a);
         }
     }
     if (mask & PMOE_PHASE_FINALIZE) {

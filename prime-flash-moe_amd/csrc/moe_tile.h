@@ -1,15 +1,14 @@
-// Device-side tile engine shared by the fused-MoE kernels (gfx950, wave64).
+// Device-side helpers shared by the fused-MoE kernels (gfx950, wave64), and the register-staged
+// tile engine of the single-group (256-thread) fused kernel; the two-group kernels of the split
+// pipeline use the ring engine in moe_ring.h.
 //
-// A workgroup of NG*256 threads (NG = 1 or 2 "token groups" of 4 waves) owns a tile of a grouped
-// GEMM whose two operands are both contiguous along the contraction dimension:
-//     NG*128 token rows (x or the activation; one 128-row sorted block per group)
-//   x 256 weight rows   (W1 or W2 of one expert, shared by the groups).
+// A workgroup of 256 threads owns a tile of a grouped GEMM whose two operands are both contiguous
+// along the contraction dimension:
+//     128 token rows (one sorted block of x, or the activation tile)
+//   x 256 weight rows (W1 or W2 of one expert).
 // The contraction is consumed in slabs of 128 bytes per row (64 bf16 or 128 e4m3), staged
 // through LDS with a double buffer: while the MFMAs of slab k run out of one buffer, the
 // global loads of slab k+1 are in flight into registers and are then written to the other.
-// With NG = 2 the two groups are two waves per SIMD working on different token rows against the
-// same weight rows: the weight slab is fetched once for 256 token rows, and one group's MFMAs
-// cover the other's LDS and barrier latencies.
 //
 // LDS layout of one stage: [NG*128 token rows][128 B] then [256 weight rows][128 B].
 // A row is 8 chunks of 16 B; chunk c of row r is stored in slot c ^ ((r >> 1) & 7), which
@@ -135,79 +134,6 @@ struct StageLoader {
             *reinterpret_cast<uint4 *>(stage + G::kTokRegion + lds_off + i * G::kPassRows * kRowBytes) = rw[i];
     }
 };
-
-// ------------------------------------------------------------------------------------------
-// Direct global -> LDS copy of one stage (global_load_lds_dwordx4): no staging registers and no
-// ds_write instructions.  A wave instruction moves 64 x 16 B = 8 consecutive LDS rows; lane l
-// writes LDS bytes [16 l, 16 l + 16) behind the wave-uniform base (M0), so the swizzle is applied
-// on the global side: the lane that lands in slot s of row r fetches chunk s ^ swz(r).
-template <int NG>
-struct DmaLoader {
-    using G = Geo<NG>;
-    const char *tok_base;
-    const char *w_base[2];
-    uint32_t tok_off[G::kTokPasses];
-    uint32_t w_off;
-    uint32_t w_pitch_pass;
-    int lds_wave_off;  // byte offset of this wave's 8 rows inside a pass (wave-uniform)
-    int tok_mask;      // token passes that hold live rows (wave-uniform)
-
-    // The copy is written as inline assembly: issued through the compiler's builtin, every later LDS
-    // read would first wait for all copies in flight (the compiler cannot tell the stage being read
-    // from the stage being filled), which would serialise copy and compute.  The hardware counter
-    // still counts these loads; wait_all() must run before the barrier that publishes a stage.
-    static __device__ __forceinline__ void copy16(const char *base, uint32_t voff, char *lds_dst) {
-        const uint32_t m0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)lds_dst;
-        asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :
-                     : "v"(voff), "s"(base), "s"(m0)
-                     : "memory");
-    }
-    static __device__ __forceinline__ void wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
-    __device__ __forceinline__ void issue(char *stage, uint32_t koff) const {
-#pragma unroll
-        for (int i = 0; i < G::kTokPasses; ++i)
-            if (tok_mask & (1 << i))
-                copy16(tok_base, tok_off[i] + koff, stage + lds_wave_off + i * G::kPassRows * kRowBytes);
-#pragma unroll
-        for (int i = 0; i < G::kWPasses; ++i)
-            copy16(w_base[i / G::kWPassesPerHalf], w_off + (i % G::kWPassesPerHalf) * w_pitch_pass + koff,
-                   stage + G::kTokRegion + lds_wave_off + i * G::kPassRows * kRowBytes);
-    }
-};
-
-// bf16 operand fragments of one 16-wide K sub-step: 2 weight fragments and up to 4 token fragments
-struct FragsBf16 {
-    bf16x8 a[2];
-    bf16x8 b[4];
-};
-
-template <int NTF>
-__device__ __forceinline__ void fetch_bf16(FragsBf16 &fr, const char *tok, const char *wgt, const int (&wrow)[2],
-                                           int lane, int j) {
-    const int r = lane & 31, half = lane >> 5, sx = (lane >> 1) & 7;
-    const int off = r * kRowBytes + (((2 * j + half) ^ sx) << 4);
-#pragma unroll
-    for (int f = 0; f < 2; ++f) fr.a[f] = *reinterpret_cast<const bf16x8 *>(wgt + wrow[f] * kRowBytes + off);
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-        if (t < NTF) fr.b[t] = *reinterpret_cast<const bf16x8 *>(tok + t * 32 * kRowBytes + off);
-}
-
-template <int NTF, bool TRANSPOSED>
-__device__ __forceinline__ void mma_bf16(f32x16 (&acc)[2][4], const FragsBf16 &fr) {
-#pragma unroll
-    for (int f = 0; f < 2; ++f)
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-            if (t < NTF) {
-                if constexpr (TRANSPOSED)
-                    acc[f][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.a[f], fr.b[t], acc[f][t], 0, 0, 0);
-                else
-                    acc[f][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.b[t], fr.a[f], acc[f][t], 0, 0, 0);
-            }
-}
 
 // ------------------------------------------------------------------------------------------
 // MFMA over one 128-byte slab.  `tok` points at this wave's group of 128 token rows, `wgt` at the

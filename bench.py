@@ -178,6 +178,9 @@ def main():
     ap.add_argument("--split", type=int, default=1)
     ap.add_argument("--all", action="store_true", help="also time every benchmark configuration (stderr)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (a kernel of known traffic, to scale the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path is single-device, "
@@ -189,6 +192,14 @@ def main():
     log = lambda *a: print(*a, file=sys.stderr, flush=True)
     log(f"device: {torch.cuda.get_device_name(0)}; peaks used: bf16 {PEAK_TFLOPS['bf16']} / "
         f"mxfp8 {PEAK_TFLOPS['mxfp8']} TFLOP/s dense, HBM {PEAK_HBM_GBS} GB/s")
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
     if args.all:
         for name, cfg in CONFIGS.items():
             if name == args.config:

@@ -36,6 +36,7 @@ struct MoeArgs {
     float *accum;         // (M, K) fp32 accumulator
     const int2 *tiles;    // row tiles built by the prologue: (first block, number of blocks 1..2)
     const int *n_tiles;   // number of row tiles
+    const int2 *work;     // this kernel's tile order: (first block | blocks << 28, weight tile)
     int top_k, M, K, N, H, E, sorted_num;
     int n_blocks;  // sorted_num / 128 (rounded up)
     int n_wtiles;  // weight tiles along the free dimension: H/128 (up) or ceil(K/256) (down)
@@ -46,10 +47,9 @@ constexpr int kActPitchFp8 = 144;   // 128 e4m3 + 16 B pad
 
 // Workgroup id -> (row tile, weight tile), using the live tile count read on the device.
 // Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; ids are regrouped so that
-// one XCD runs a contiguous range of logical ids, and a range is walked as
-// [group of GW weight tiles][row tiles][weight tile in group]: the ~32 tiles resident on an XCD
-// then share their token rows GW ways and, for experts spanning several row tiles, their weight
-// slice several ways inside that XCD's L2.
+// one XCD runs a contiguous range of logical ids.  The two-group kernels then look their tile up in
+// the work list the prologue built (expert-major order, see moe_prologue_kernel); the single-group
+// fused kernel walks [group of 8 weight tiles][row blocks][weight tile in group].
 template <int NG>
 __device__ __forceinline__ bool resolve_tile(const MoeArgs &a, int &first, int &nb, int &wt) {
     int n_row_tiles;
@@ -61,27 +61,26 @@ __device__ __forceinline__ bool resolve_tile(const MoeArgs &a, int &first, int &
     if (idx >= per_xcd) return false;
     const int logical = (int)(blockIdx.x & 7) * per_xcd + idx;
     if (logical >= G) return false;
-    constexpr int GW = 8;
-    const int full = a.n_wtiles / GW * GW;
-    const int per_group = n_row_tiles * GW;
-    const int g = logical / per_group;
-    int rt;
-    if (g * GW < full) {
-        const int rem = logical - g * per_group;
-        rt = rem / GW;
-        wt = g * GW + rem % GW;
-    } else {
-        const int tw = a.n_wtiles - full;
-        const int rem = logical - (full / GW) * per_group;
-        rt = rem / tw;
-        wt = full + rem % tw;
-    }
     if constexpr (NG == 2) {
-        const int2 t = a.tiles[rt];
-        first = t.x;
-        nb = t.y;
+        const int2 w = a.work[logical];
+        first = w.x & 0x0fffffff;
+        nb = w.x >> 28;
+        wt = w.y;
     } else {
-        first = rt;
+        constexpr int GW = 8;
+        const int full = a.n_wtiles / GW * GW;
+        const int per_group = n_row_tiles * GW;
+        const int g = logical / per_group;
+        if (g * GW < full) {
+            const int rem = logical - g * per_group;
+            first = rem / GW;
+            wt = g * GW + rem % GW;
+        } else {
+            const int tw = a.n_wtiles - full;
+            const int rem = logical - (full / GW) * per_group;
+            first = rem / tw;
+            wt = full + rem % tw;
+        }
         nb = 1;
     }
     return true;
@@ -610,12 +609,30 @@ __global__ __launch_bounds__(256) void moe_fused_kernel(MoeArgs a) {
     }
 }
 
-// Prologue of every call: clears the fp32 accumulator and (workgroup 0) builds the list of row
-// tiles for the two-group kernels: consecutive blocks of one expert are paired, an expert's odd
-// last block stays single.  One pass of block-wide scans per 256 blocks.
+// Walk order of the tiles of one kernel.  Row tiles of one expert are consecutive in `tiles`; an
+// expert with T row tiles and a kernel with n_wt weight tiles own T * n_wt consecutive work items,
+// ordered [group of 8 weight tiles][row tile of the expert][weight tile in group].  The ~32
+// workgroups that run side by side on an XCD are then (a few row tiles of ONE expert) x (8 weight
+// tiles): every weight slab they fetch is shared by all the expert's row tiles and every token
+// slab by 8 weight tiles, inside that XCD's L2.
+__device__ __forceinline__ void emit_work(int2 *work, int n_wt, int tile, int q, int T, int first, int nb) {
+    constexpr int GW = 8;
+    const int base = (tile - q) * n_wt;  // first work item of the expert
+    for (int wt = 0; wt < n_wt; ++wt) {
+        const int wg = wt / GW;
+        const int gw = min(GW, n_wt - wg * GW);
+        work[base + wg * GW * T + q * gw + (wt - wg * GW)] = make_int2(first | (nb << 28), wt);
+    }
+}
+
+// Prologue of every call: clears the fp32 accumulator and (workgroup 0) builds the row tiles and
+// work lists of the two-group kernels: consecutive blocks of one expert are paired, an expert's odd
+// last block stays single.  One pass of block-wide scans per 256 blocks, then one pass over the
+// tiles that finds each expert's tile count by bisection and writes the two walk orders.
 __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert_ids, const int32_t *ntpp,
-                                                           int n_blocks, int2 *tiles, int *n_tiles,
-                                                           float4 *accum, int64_t n4, int do_zero) {
+                                                           int n_blocks, int2 *tiles, int *tile_run, int *n_tiles,
+                                                           int2 *work_up, int n_wt_up, int2 *work_down,
+                                                           int n_wt_down, float4 *accum, int64_t n4, int do_zero) {
     if (blockIdx.x == 0 && tiles != nullptr) {
         __shared__ int s_max[4], s_sum[4], s_carry[2];
         const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -650,12 +667,32 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
             __syncthreads();
             int off = s_carry[1];
             for (int w = 0; w < wave; ++w) off += s_sum[w];
-            if (leader) tiles[off + incl - 1] = make_int2(b, paired ? 2 : 1);
+            if (leader) {
+                tiles[off + incl - 1] = make_int2(b, paired ? 2 : 1);
+                tile_run[off + incl - 1] = run_start;
+            }
             __syncthreads();
             if (tid == 255) { s_carry[0] = run_start; s_carry[1] = off + incl; }
             __syncthreads();
         }
-        if (tid == 0) n_tiles[0] = s_carry[1];
+        const int nt = s_carry[1];
+        if (tid == 0) n_tiles[0] = nt;
+        __threadfence_block();
+        __syncthreads();  // tiles / tile_run written above are read below by other threads
+        for (int t = tid; t < nt; t += 256) {
+            const int2 tl = tiles[t];
+            const int rs = tile_run[t];
+            const int q = (tl.x - rs) >> 1;  // index of the tile inside its expert
+            int lo = t, hi = nt - 1;         // last tile of the same run (tile_run is non-decreasing)
+            while (lo < hi) {
+                const int mid = (lo + hi + 1) >> 1;
+                if (tile_run[mid] == rs) lo = mid;
+                else hi = mid - 1;
+            }
+            const int T = lo - (t - q) + 1;
+            emit_work(work_up, n_wt_up, t, q, T, tl.x, tl.y);
+            emit_work(work_down, n_wt_down, t, q, T, tl.x, tl.y);
+        }
     }
     if (do_zero) {
         const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -690,18 +727,25 @@ __global__ __launch_bounds__(256) void finalize_kernel(const float4 *acc, uint4 
 // ------------------------------------------------------------------------------------------ host
 
 struct WorkspaceLayout {
-    size_t n_tiles_off, tiles_off, accum_off, act_off, act_scales_off, total;
+    size_t n_tiles_off, tiles_off, tile_run_off, work_up_off, work_down_off, accum_off, act_off, act_scales_off, total;
 };
 
 static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_num, int split) {
     WorkspaceLayout l{};
     const size_t H = (size_t)N / 2;
     const size_t rows = align_up((size_t)sorted_num, kBlockRows);
+    const size_t blocks = rows / kBlockRows;
     size_t off = 0;
     l.n_tiles_off = off;
     off += 256;
     l.tiles_off = off;
-    off = align_up(off + (rows / kBlockRows) * sizeof(int2), 256);
+    off = align_up(off + blocks * sizeof(int2), 256);
+    l.tile_run_off = off;
+    off = align_up(off + blocks * sizeof(int), 256);
+    l.work_up_off = off;
+    if (split) off = align_up(off + blocks * (H / 128) * sizeof(int2), 256);
+    l.work_down_off = off;
+    if (split) off = align_up(off + blocks * (((size_t)K + kWRows - 1) / kWRows) * sizeof(int2), 256);
     l.accum_off = off;
     off = align_up(off + (size_t)M * K * sizeof(float), 256);
     l.act_off = off;
@@ -721,28 +765,41 @@ static int grid_for(int n_tiles) { return (n_tiles + 7) / 8 * 8; }
 // pmoe_set_phase_mask in the header.
 static thread_local int g_phase_mask = PMOE_PHASE_ALL;
 
+struct SchedBuffers {
+    int2 *tiles;
+    int *tile_run;
+    int *n_tiles;
+    int2 *work_up;
+    int2 *work_down;
+};
+
 template <int DT>
-static int launch_pipeline(MoeArgs a, void *out, int split, hipStream_t s) {
+static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int split, hipStream_t s) {
     const int64_t n_out = (int64_t)a.M * a.K;  // K % 128 == 0, so n_out % 8 == 0
     const int mask = g_phase_mask;
     a.n_blocks = (a.sorted_num + kBlockRows - 1) / kBlockRows;
     a.n_wtiles = a.H / 128;
+    a.tiles = sb.tiles;
+    a.n_tiles = sb.n_tiles;
+    const int n_wt_down = (a.K + kWRows - 1) / kWRows;
     {
-        // the tile list is needed by the two-group kernels even when the clear is masked off
+        // the tile lists are needed by the two-group kernels even when the clear is masked off
         const int64_t n4 = n_out / 4;
         const int do_zero = (mask & PMOE_PHASE_ZERO) ? 1 : 0;
         const int blocks = do_zero ? (int)std::min<int64_t>((n4 + 255) / 256, 2048) : 1;
         hipLaunchKernelGGL(moe_prologue_kernel, dim3(blocks), dim3(256), 0, s, a.expert_ids, a.ntpp, a.n_blocks,
-                           split ? const_cast<int2 *>(a.tiles) : nullptr, const_cast<int *>(a.n_tiles),
-                           reinterpret_cast<float4 *>(a.accum), n4, do_zero);
+                           split ? sb.tiles : nullptr, sb.tile_run, sb.n_tiles, sb.work_up, a.n_wtiles,
+                           sb.work_down, n_wt_down, reinterpret_cast<float4 *>(a.accum), n4, do_zero);
     }
     if (a.n_blocks > 0) {
         const int grid = grid_for(a.n_blocks * a.n_wtiles);
         if (split) {
+            a.work = sb.work_up;
             if (mask & PMOE_PHASE_UP)
                 hipLaunchKernelGGL((moe_up_kernel<DT>), dim3(grid), dim3(512), 0, s, a);
             MoeArgs d = a;
-            d.n_wtiles = (a.K + kWRows - 1) / kWRows;
+            d.n_wtiles = n_wt_down;
+            d.work = sb.work_down;
             if (mask & PMOE_PHASE_DOWN)
                 hipLaunchKernelGGL((moe_down_kernel<DT>), dim3(grid_for(d.n_blocks * d.n_wtiles)), dim3(512), 0, s, d);
         } else if (mask & PMOE_PHASE_UP) {
@@ -760,6 +817,16 @@ static int launch_pipeline(MoeArgs a, void *out, int split, hipStream_t s) {
                                reinterpret_cast<const float4 *>(a.accum), reinterpret_cast<uint4 *>(out), n8);
     }
     return check_launch("fused_moe launch");
+}
+
+static SchedBuffers sched_buffers(char *ws, const WorkspaceLayout &l) {
+    SchedBuffers sb;
+    sb.n_tiles = reinterpret_cast<int *>(ws + l.n_tiles_off);
+    sb.tiles = reinterpret_cast<int2 *>(ws + l.tiles_off);
+    sb.tile_run = reinterpret_cast<int *>(ws + l.tile_run_off);
+    sb.work_up = reinterpret_cast<int2 *>(ws + l.work_up_off);
+    sb.work_down = reinterpret_cast<int2 *>(ws + l.work_down_off);
+    return sb;
 }
 
 }  // namespace pmoe
@@ -818,12 +885,10 @@ extern "C" int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2,
     a.ntpp = num_tokens_post_padded;
     a.topk_w = topk_weights;
     char *ws = static_cast<char *>(workspace);
-    a.n_tiles = reinterpret_cast<const int *>(ws + l.n_tiles_off);
-    a.tiles = reinterpret_cast<const int2 *>(ws + l.tiles_off);
     a.accum = reinterpret_cast<float *>(ws + l.accum_off);
     a.act = ws + l.act_off;
     a.top_k = top_k; a.M = M; a.K = K; a.N = N; a.H = N / 2; a.E = num_experts; a.sorted_num = sorted_num;
-    return launch_pipeline<DT_BF16>(a, out, split, static_cast<hipStream_t>(stream));
+    return launch_pipeline<DT_BF16>(a, sched_buffers(ws, l), out, split, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int pmoe_fused_moe_mxfp8(const void *x, const void *x_scales, const void *w,
@@ -858,11 +923,9 @@ extern "C" int pmoe_fused_moe_mxfp8(const void *x, const void *x_scales, const v
     a.ntpp = num_tokens_post_padded;
     a.topk_w = topk_weights;
     char *ws = static_cast<char *>(workspace);
-    a.n_tiles = reinterpret_cast<const int *>(ws + l.n_tiles_off);
-    a.tiles = reinterpret_cast<const int2 *>(ws + l.tiles_off);
     a.accum = reinterpret_cast<float *>(ws + l.accum_off);
     a.act = ws + l.act_off;
     a.act_scales = reinterpret_cast<uint8_t *>(ws + l.act_scales_off);
     a.top_k = top_k; a.M = M; a.K = K; a.N = N; a.H = N / 2; a.E = num_experts; a.sorted_num = sorted_num;
-    return launch_pipeline<DT_FP8>(a, out, split, static_cast<hipStream_t>(stream));
+    return launch_pipeline<DT_FP8>(a, sched_buffers(ws, l), out, split, static_cast<hipStream_t>(stream));
 }

@@ -193,10 +193,12 @@ def main():
     log(f"device: {torch.cuda.get_device_name(0)}; peaks used: bf16 {PEAK_TFLOPS['bf16']} / "
         f"mxfp8 {PEAK_TFLOPS['mxfp8']} TFLOP/s dense, HBM {PEAK_HBM_GBS} GB/s")
     if args.calibrate_copy:
+        from prime_moe import _native
         src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
         dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        for _ in range(3):  # copy_calibration_kernel: reads 1 GiB, writes 1 GiB
+            _native.check(_native.load().pmoe_copy_calibration(src.data_ptr(), dst.data_ptr(), src.numel() * 4,
+                                                               torch.cuda.current_stream().cuda_stream))
         torch.cuda.synchronize()
         del src, dst
         torch.cuda.empty_cache()

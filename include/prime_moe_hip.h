@@ -120,6 +120,14 @@ int pmoe_quantize_mx(const void *src_bf16, void *q, void *scales, int64_t rows, 
 #define PMOE_PHASE_ALL 15
 void pmoe_set_phase_mask(int mask);
 
+/*
+ * Second profiling aid without a counterpart in the reference: a plain device copy of `bytes`
+ * bytes (multiple of 16) done by a kernel named copy_calibration_kernel.  Its known traffic
+ * (bytes read, bytes written) scales the FETCH_SIZE / WRITE_SIZE hardware counters of a
+ * counter-collection run that also contains the fused kernels.
+ */
+int pmoe_copy_calibration(const void *src, void *dst, int64_t bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -258,31 +258,68 @@ __device__ __forceinline__ void store_act_tile(const MoeArgs &a, const char *til
 // ==========================================================================================
 
 // Common set-up of the ring loader.  Token rows: `tok_row_off(row)` gives the byte offset of tile
-// row `row` (0..255) in `tok_base`; weight rows: the tile's two 128-row halves start at w_base[0/1]
-// with `w_pitch` bytes per row.  Scales (mxfp8): `tok_sc_off(row)` / `w_sc_off(row)` are the byte
-// offsets of the row's first 4-scale dword.
-template <int DT, typename TokOff, typename TokScOff, typename WScOff>
-__device__ __forceinline__ void setup_ring_loader(ring::Loader &ld, int tid, uint32_t w_pitch, TokOff tok_row_off,
-                                                  const uint8_t *tok_sc_base, TokScOff tok_sc_off,
-                                                  const uint8_t *w_sc_base, WScOff w_sc_off) {
-    const int wave = tid >> 6, lane = tid & 63;
-    const int prow = tid >> 2;                      // row inside a 128-row pass
+// row `row` in `tok_base`; weight rows: the tile's two 128-row halves start at w_base[0/1] with
+// `w_pitch` bytes per row.  Scales (mxfp8): `tok_sc_off(row)` / `w_sc_off(row)` are the byte offsets
+// of the row's first 4-scale dword.  ntf0 / ntf1 = 32-row fragments with live rows in the two
+// blocks of the tile; token rows (and their scales) of dead fragments are not copied.
+template <int DT, bool SKINNY, typename TokOff, typename TokScOff, typename WScOff>
+__device__ __forceinline__ void setup_ring_loader(ring::Loader &ld, int tid, uint32_t w_pitch, int ntf0, int ntf1,
+                                                  TokOff tok_row_off, const uint8_t *tok_sc_base,
+                                                  TokScOff tok_sc_off, const uint8_t *w_sc_base, WScOff w_sc_off) {
+    using C = ring::Cfg<DT, SKINNY>;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int prow = tid >> 2;                         // row inside a 128-row pass
     const int gchunk = (tid & 3) ^ ring::swz64(prow);  // global chunk landing in this lane's LDS slot
-    ld.tok_off[0] = tok_row_off(prow) + gchunk * 16;
-    ld.tok_off[1] = tok_row_off(kBlockRows + prow) + gchunk * 16;
     ld.w_off = (uint32_t)prow * w_pitch + gchunk * 16;
-    ld.wave_off = __builtin_amdgcn_readfirstlane(wave * 16 * ring::kRB);
-    ld.wave_sc_off = __builtin_amdgcn_readfirstlane(wave * 64 * 4);
+    ld.w_dst[0] = C::kTokRegion + wave * 16 * ring::kRB;
+    ld.w_dst[1] = ld.w_dst[0] + 128 * ring::kRB;
+    ld.tok_dst[0] = ld.tok_dst[1] = -1;
+    ld.tok_off[0] = ld.tok_off[1] = 0;
+    if constexpr (SKINNY) {
+        if (wave < 2) {  // 32 rows = two wave instructions
+            ld.tok_dst[0] = wave * 16 * ring::kRB;
+            ld.tok_off[0] = tok_row_off(prow) + gchunk * 16;
+        }
+    } else {
+        const int frag = wave >> 1;  // the wave's 16 rows of a block lie in this fragment
+        if (frag < ntf0) {
+            ld.tok_dst[0] = wave * 16 * ring::kRB;
+            ld.tok_off[0] = tok_row_off(prow) + gchunk * 16;
+        }
+        if (frag < ntf1) {
+            ld.tok_dst[1] = ring::kGroupRegion + wave * 16 * ring::kRB;
+            ld.tok_off[1] = tok_row_off(kBlockRows + prow) + gchunk * 16;
+        }
+    }
     ld.sc_base = nullptr;
     ld.sc_off = 0;
     ld.sc_step = 0;
+    ld.sc_dst = -1;
     if constexpr (DT == DT_FP8) {
-        const int row = wave * 64 + lane;  // 0..255 token rows, 256..511 weight rows
-        const bool is_tok = __builtin_amdgcn_readfirstlane(wave) < 4;
-        ld.sc_base = reinterpret_cast<const char *>(is_tok ? tok_sc_base : w_sc_base);
-        ld.sc_off = is_tok ? tok_sc_off(row) : w_sc_off(row - ring::kTokRows);
-        ld.sc_step = is_tok ? 4u : 512u;
+        if (wave >= 4) {  // weight rows 64 (wave - 4) + lane
+            const int row = 64 * (wave - 4) + lane;
+            ld.sc_base = reinterpret_cast<const char *>(w_sc_base);
+            ld.sc_off = w_sc_off(row);
+            ld.sc_step = 512u;
+            ld.sc_dst = C::kScaleOff + (C::kScaleTokRows + 64 * (wave - 4)) * 4;
+        } else if constexpr (SKINNY) {
+            if (wave == 2) {  // token rows 0..31 (the upper lanes repeat row 31 into unused dwords)
+                ld.sc_base = reinterpret_cast<const char *>(tok_sc_base);
+                ld.sc_off = tok_sc_off(min(lane, 31));
+                ld.sc_step = 4u;
+                ld.sc_dst = C::kScaleOff;
+            }
+        } else {
+            const int row = 64 * wave + lane;  // token rows: block wave / 2, fragments 2 (wave & 1), + 1
+            if (2 * (wave & 1) < ((wave >> 1) ? ntf1 : ntf0)) {
+                ld.sc_base = reinterpret_cast<const char *>(tok_sc_base);
+                ld.sc_off = tok_sc_off(row);
+                ld.sc_step = 4u;
+                ld.sc_dst = C::kScaleOff + 64 * wave * 4;
+            }
+        }
     }
+    ld.lps = 2 + (ld.tok_dst[0] >= 0) + (ld.tok_dst[1] >= 0) + (ld.sc_dst >= 0);
 }
 
 // First slab of this workgroup's walk over K: workgroups that run side by side on an XCD (consecutive
@@ -292,10 +329,11 @@ __device__ __forceinline__ int slab_rotation(int n_slabs) {
     return phase % n_slabs & ~1;
 }
 
-// Up kernel tile: NG = 2 row blocks x activation columns [128 ht, 128 ht + 128).  LDS weight rows
-// 0..127 are gate rows, 128..255 the matching up rows; wave v of a group owns gate/up rows
-// 32v..32v+31 so gate and up of one activation element sit in the same lane and register.
-template <int DT, int NTF>
+// Up kernel tile: two row blocks (SKINNY: one block with at most 32 live rows) x activation columns
+// [128 ht, 128 ht + 128).  LDS weight rows 0..127 are gate rows, 128..255 the matching up rows; wave
+// v of a group owns gate/up rows 32v..32v+31 so gate and up of one activation element sit in the
+// same lane and register.
+template <int DT, bool SKINNY, int NTF, bool FULL>
 __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht, int e, RowInfo<2> &ri,
                                              char *lds, uint32_t *act_sc_lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
@@ -303,7 +341,9 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
     const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
     const int K = a.K, H = a.H, N = a.N;
     const int h0 = ht * 128;
-    const int my_ntf = __builtin_amdgcn_readfirstlane((ri.nvalid[grp] + 31) >> 5);
+    const int ntf0 = __builtin_amdgcn_readfirstlane((ri.nvalid[0] + 31) >> 5);
+    const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
+    const int my_ntf = grp ? ntf1 : ntf0;
     const bool active = my_ntf > 0;
 
     ring::Loader ld;
@@ -312,8 +352,8 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
     ld.w_base[1] = ld.w_base[0] + (int64_t)H * K * ES;
     const uint32_t row_bytes = (uint32_t)(K * ES);
     const int kb = K >> 5;
-    setup_ring_loader<DT>(
-        ld, tid, row_bytes,
+    setup_ring_loader<DT, SKINNY>(
+        ld, tid, row_bytes, ntf0, ntf1,
         [&](int row) { return (uint32_t)max(ri.tok[row], 0) * row_bytes; },  // dead rows read token 0
         a.x_scales, [&](int row) { return (uint32_t)max(ri.tok[row], 0) * (uint32_t)kb; },
         a.w1_scales + (int64_t)e * N * kb,
@@ -324,8 +364,9 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
     zero_acc(acc);
     const int n_slabs = (K * ES) / ring::kRB;
     const int start = slab_rotation(n_slabs);
-    if (active) ring::main_loop<DT, NTF, true, true>(acc, ld, lds, n_slabs, wrow, lane, grp, start);
-    else ring::main_loop<DT, NTF, true, false>(acc, ld, lds, n_slabs, wrow, lane, grp, start);
+    const int tok_region = SKINNY ? 0 : grp * ring::kGroupRegion;
+    if (active) ring::main_loop<DT, SKINNY, NTF, true, true, FULL>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
+    else ring::main_loop<DT, SKINNY, NTF, true, false, FULL>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
 
     // the ring is free (main_loop ends with a barrier): reuse it for the activation tiles
     constexpr int kPitch = DT == DT_BF16 ? kActPitchBf16 : kActPitchFp8;
@@ -338,7 +379,7 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
 
 template <int DT>
 __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
-    __shared__ __attribute__((aligned(1024))) char lds[ring::kStages * ring::stage_bytes<DT>()];
+    __shared__ __attribute__((aligned(1024))) char lds[ring::ring_bytes<DT>()];
     __shared__ uint32_t act_sc_lds[kBlockRows * 2];
     __shared__ RowInfo<2> ri;
     int first, nb, ht;
@@ -348,14 +389,17 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
     if (ntf == 0) return;
     const int e = a.expert_ids[first];
     if (e < 0 || e >= a.E) return;
-    if (ntf == 1) up_tile_ring<DT, 1>(a, first, ht, e, ri, lds, act_sc_lds);
-    else if (ntf == 2) up_tile_ring<DT, 2>(a, first, ht, e, ri, lds, act_sc_lds);
-    else up_tile_ring<DT, 4>(a, first, ht, e, ri, lds, act_sc_lds);
+    const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
+    if (ntf == 1 && ri.nvalid[1] == 0) up_tile_ring<DT, true, 1, false>(a, first, ht, e, ri, lds, act_sc_lds);
+    else if (ntf == 1) up_tile_ring<DT, false, 1, false>(a, first, ht, e, ri, lds, act_sc_lds);
+    else if (ntf == 2) up_tile_ring<DT, false, 2, false>(a, first, ht, e, ri, lds, act_sc_lds);
+    else if (full) up_tile_ring<DT, false, 4, true>(a, first, ht, e, ri, lds, act_sc_lds);
+    else up_tile_ring<DT, false, 4, false>(a, first, ht, e, ri, lds, act_sc_lds);
 }
 
 // Down kernel of the split pipeline: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
 // full reduction over H inside the workgroup (no split-K), then w[row] * y added to accum[token].
-template <int DT, int NTF>
+template <int DT, bool SKINNY, int NTF, bool FULL>
 __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, char *lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -363,7 +407,9 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     const int K = a.K, H = a.H;
     const int k0 = kt * kWRows;
     const int64_t row0 = (int64_t)first * kBlockRows;
-    const bool active = __builtin_amdgcn_readfirstlane(ri.nvalid[grp]) > 0;
+    const int ntf0 = __builtin_amdgcn_readfirstlane((ri.nvalid[0] + 31) >> 5);
+    const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
+    const bool active = (grp ? ntf1 : ntf0) > 0;
 
     ring::Loader ld;
     ld.tok_base = a.act + row0 * H * ES;
@@ -371,11 +417,9 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     ld.w_base[1] = (k0 + 128 < K) ? ld.w_base[0] + (int64_t)128 * H * ES : ld.w_base[0];
     const uint32_t row_bytes = (uint32_t)(H * ES);
     const int hb = H >> 5;
-    // rows of a block that does not belong to this tile (single tiles) re-read the tile's row 0
-    const int live_rows = __builtin_amdgcn_readfirstlane(ri.nvalid[1] > 0 ? 2 * kBlockRows : kBlockRows);
-    setup_ring_loader<DT>(
-        ld, tid, row_bytes, [&](int row) { return (uint32_t)(row < live_rows ? row : 0) * row_bytes; },
-        a.act_scales + row0 * hb, [&](int row) { return (uint32_t)(row < live_rows ? row : 0) * (uint32_t)hb; },
+    setup_ring_loader<DT, SKINNY>(
+        ld, tid, row_bytes, ntf0, ntf1, [&](int row) { return (uint32_t)row * row_bytes; },
+        a.act_scales + row0 * hb, [&](int row) { return (uint32_t)row * (uint32_t)hb; },
         a.w2_scales + (int64_t)e * K * hb,
         [&](int row) { return (uint32_t)blocked_scale_off(min(k0 + row, K - 1), 0, H >> 7); });
 
@@ -384,17 +428,18 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     zero_acc(acc);
     const int n_slabs = (H * ES) / ring::kRB;
     const int start = slab_rotation(n_slabs);
+    const int tok_region = SKINNY ? 0 : grp * ring::kGroupRegion;
     if (active) {
-        ring::main_loop<DT, NTF, false, true>(acc, ld, lds, n_slabs, wrow, lane, grp, start);
+        ring::main_loop<DT, SKINNY, NTF, false, true, FULL>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
         scatter_add<NTF>(acc, ri.tok + grp * kBlockRows, ri.wt + grp * kBlockRows, a.accum, K, k0 + 64 * w4, lane);
     } else {
-        ring::main_loop<DT, NTF, false, false>(acc, ld, lds, n_slabs, wrow, lane, grp, start);
+        ring::main_loop<DT, SKINNY, NTF, false, false, FULL>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
     }
 }
 
 template <int DT>
 __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
-    __shared__ __attribute__((aligned(1024))) char lds[ring::kStages * ring::stage_bytes<DT>()];
+    __shared__ __attribute__((aligned(1024))) char lds[ring::ring_bytes<DT>()];
     __shared__ RowInfo<2> ri;
     int first, nb, kt;
     if (!resolve_tile<2>(a, first, nb, kt)) return;
@@ -403,9 +448,12 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
     if (ntf == 0) return;
     const int e = a.expert_ids[first];
     if (e < 0 || e >= a.E) return;
-    if (ntf == 1) down_tile_ring<DT, 1>(a, first, kt, e, ri, lds);
-    else if (ntf == 2) down_tile_ring<DT, 2>(a, first, kt, e, ri, lds);
-    else down_tile_ring<DT, 4>(a, first, kt, e, ri, lds);
+    const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
+    if (ntf == 1 && ri.nvalid[1] == 0) down_tile_ring<DT, true, 1, false>(a, first, kt, e, ri, lds);
+    else if (ntf == 1) down_tile_ring<DT, false, 1, false>(a, first, kt, e, ri, lds);
+    else if (ntf == 2) down_tile_ring<DT, false, 2, false>(a, first, kt, e, ri, lds);
+    else if (full) down_tile_ring<DT, false, 4, true>(a, first, kt, e, ri, lds);
+    else down_tile_ring<DT, false, 4, false>(a, first, kt, e, ri, lds);
 }
 
 // ==========================================================================================
@@ -609,28 +657,27 @@ __global__ __launch_bounds__(256) void moe_fused_kernel(MoeArgs a) {
     }
 }
 
-// Walk order of the tiles of one kernel.  Row tiles of one expert are consecutive in `tiles`; an
-// expert with T row tiles and a kernel with n_wt weight tiles own T * n_wt consecutive work items,
-// ordered [group of 8 weight tiles][row tile of the expert][weight tile in group].  The ~32
-// workgroups that run side by side on an XCD are then (a few row tiles of ONE expert) x (8 weight
-// tiles): every weight slab they fetch is shared by all the expert's row tiles and every token
-// slab by 8 weight tiles, inside that XCD's L2.
-__device__ __forceinline__ void emit_work(int2 *work, int n_wt, int tile, int q, int T, int first, int nb) {
+// Walk order of the tiles of one kernel: [group of 8 weight tiles][row tile][weight tile in group].
+// The ~32 workgroups that run side by side on an XCD are then 4 consecutive row tiles (mostly of one
+// expert) x 8 weight tiles: every token slab they fetch is shared by 8 weight tiles and every weight
+// slab by the row tiles of its expert, inside that XCD's L2.  (Walking expert by expert instead,
+// so that all row tiles of an expert always meet, measured 5 % slower on the Mixtral-like shape:
+// more workgroups then ask for the same lines at the same moment.)
+__device__ __forceinline__ void emit_work(int2 *work, int n_wt, int tile, int n_tiles, int first, int nb) {
     constexpr int GW = 8;
-    const int base = (tile - q) * n_wt;  // first work item of the expert
     for (int wt = 0; wt < n_wt; ++wt) {
         const int wg = wt / GW;
         const int gw = min(GW, n_wt - wg * GW);
-        work[base + wg * GW * T + q * gw + (wt - wg * GW)] = make_int2(first | (nb << 28), wt);
+        work[wg * GW * n_tiles + tile * gw + (wt - wg * GW)] = make_int2(first | (nb << 28), wt);
     }
 }
 
 // Prologue of every call: clears the fp32 accumulator and (workgroup 0) builds the row tiles and
 // work lists of the two-group kernels: consecutive blocks of one expert are paired, an expert's odd
 // last block stays single.  One pass of block-wide scans per 256 blocks, then one pass over the
-// tiles that finds each expert's tile count by bisection and writes the two walk orders.
+// tiles that writes the two walk orders.
 __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert_ids, const int32_t *ntpp,
-                                                           int n_blocks, int2 *tiles, int *tile_run, int *n_tiles,
+                                                           int n_blocks, int2 *tiles, int *n_tiles,
                                                            int2 *work_up, int n_wt_up, int2 *work_down,
                                                            int n_wt_down, float4 *accum, int64_t n4, int do_zero) {
     if (blockIdx.x == 0 && tiles != nullptr) {
@@ -667,10 +714,7 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
             __syncthreads();
             int off = s_carry[1];
             for (int w = 0; w < wave; ++w) off += s_sum[w];
-            if (leader) {
-                tiles[off + incl - 1] = make_int2(b, paired ? 2 : 1);
-                tile_run[off + incl - 1] = run_start;
-            }
+            if (leader) tiles[off + incl - 1] = make_int2(b, paired ? 2 : 1);
             __syncthreads();
             if (tid == 255) { s_carry[0] = run_start; s_carry[1] = off + incl; }
             __syncthreads();
@@ -678,20 +722,11 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
         const int nt = s_carry[1];
         if (tid == 0) n_tiles[0] = nt;
         __threadfence_block();
-        __syncthreads();  // tiles / tile_run written above are read below by other threads
+        __syncthreads();  // tiles written above are read below by other threads
         for (int t = tid; t < nt; t += 256) {
             const int2 tl = tiles[t];
-            const int rs = tile_run[t];
-            const int q = (tl.x - rs) >> 1;  // index of the tile inside its expert
-            int lo = t, hi = nt - 1;         // last tile of the same run (tile_run is non-decreasing)
-            while (lo < hi) {
-                const int mid = (lo + hi + 1) >> 1;
-                if (tile_run[mid] == rs) lo = mid;
-                else hi = mid - 1;
-            }
-            const int T = lo - (t - q) + 1;
-            emit_work(work_up, n_wt_up, t, q, T, tl.x, tl.y);
-            emit_work(work_down, n_wt_down, t, q, T, tl.x, tl.y);
+            emit_work(work_up, n_wt_up, t, nt, tl.x, tl.y);
+            emit_work(work_down, n_wt_down, t, nt, tl.x, tl.y);
         }
     }
     if (do_zero) {
@@ -727,7 +762,7 @@ __global__ __launch_bounds__(256) void finalize_kernel(const float4 *acc, uint4 
 // ------------------------------------------------------------------------------------------ host
 
 struct WorkspaceLayout {
-    size_t n_tiles_off, tiles_off, tile_run_off, work_up_off, work_down_off, accum_off, act_off, act_scales_off, total;
+    size_t n_tiles_off, tiles_off, work_up_off, work_down_off, accum_off, act_off, act_scales_off, total;
 };
 
 static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_num, int split) {
@@ -740,8 +775,6 @@ static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_
     off += 256;
     l.tiles_off = off;
     off = align_up(off + blocks * sizeof(int2), 256);
-    l.tile_run_off = off;
-    off = align_up(off + blocks * sizeof(int), 256);
     l.work_up_off = off;
     if (split) off = align_up(off + blocks * (H / 128) * sizeof(int2), 256);
     l.work_down_off = off;
@@ -767,7 +800,6 @@ static thread_local int g_phase_mask = PMOE_PHASE_ALL;
 
 struct SchedBuffers {
     int2 *tiles;
-    int *tile_run;
     int *n_tiles;
     int2 *work_up;
     int2 *work_down;
@@ -788,7 +820,7 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
         const int do_zero = (mask & PMOE_PHASE_ZERO) ? 1 : 0;
         const int blocks = do_zero ? (int)std::min<int64_t>((n4 + 255) / 256, 2048) : 1;
         hipLaunchKernelGGL(moe_prologue_kernel, dim3(blocks), dim3(256), 0, s, a.expert_ids, a.ntpp, a.n_blocks,
-                           split ? sb.tiles : nullptr, sb.tile_run, sb.n_tiles, sb.work_up, a.n_wtiles,
+                           split ? sb.tiles : nullptr, sb.n_tiles, sb.work_up, a.n_wtiles,
                            sb.work_down, n_wt_down, reinterpret_cast<float4 *>(a.accum), n4, do_zero);
     }
     if (a.n_blocks > 0) {
@@ -823,7 +855,6 @@ static SchedBuffers sched_buffers(char *ws, const WorkspaceLayout &l) {
     SchedBuffers sb;
     sb.n_tiles = reinterpret_cast<int *>(ws + l.n_tiles_off);
     sb.tiles = reinterpret_cast<int2 *>(ws + l.tiles_off);
-    sb.tile_run = reinterpret_cast<int *>(ws + l.tile_run_off);
     sb.work_up = reinterpret_cast<int2 *>(ws + l.work_up_off);
     sb.work_down = reinterpret_cast<int2 *>(ws + l.work_down_off);
     return sb;

@@ -1,45 +1,56 @@
-// Ring engine of the two-group (512-thread) grouped-GEMM kernels, gfx950.
+// Ring engine of the 512-thread grouped-GEMM kernels of the split pipeline, gfx950.
 //
-// Tile: 256 token rows (two sorted blocks, one per group of 4 waves) x 256 weight rows.
-// The contraction is consumed in slabs of 64 bytes per row (32 bf16 / 64 e4m3).  Slabs are copied
-// global -> LDS by the direct-to-LDS path (global_load_lds_*: no staging registers, no ds_write)
-// into a ring of 4 stages; three slabs are in flight while one is consumed, which is what hides
-// the ~1.5 us that a burst of copies needs to drain through the vector L1 and come back from
-// L2/HBM.  One barrier per slab.
+// Tile: token rows x 256 weight rows.  The contraction is consumed in slabs of 64 bytes per row
+// (32 bf16 / 64 e4m3).  Slabs are copied global -> LDS by the direct-to-LDS path
+// (global_load_lds_*: no staging registers, no ds_write) into a ring of stages; all but one stage
+// are in flight while one is consumed.  One barrier per slab.
 //
-// Stage layout (32 KB, + 2 KB for mxfp8):
-//   [256 token rows][64 B] [256 weight rows][64 B] [512 scale dwords]
+// Two layouts of the ring share the code:
+//   WIDE   256 token rows (two sorted blocks, one per group of 4 waves), 4 stages of 32 KB (+2 KB
+//          of scales for mxfp8): the compute-bound shapes; 96 KB in flight per CU.
+//   SKINNY 32 token rows (a single block with at most 32 live rows: decode), 8 stages of 18 KB
+//          (+1.25 KB): the tile is almost only weights, and seven stages = 126 KB of weight rows in
+//          flight per CU are what it takes to keep HBM busy (latency x bandwidth per CU ~ 60 KB).
+//
+// Stage layout: [token rows][64 B] [256 weight rows][64 B] [scale dwords of all rows (mxfp8)].
 // A row is 4 chunks of 16 B; chunk c of row r sits in slot c ^ ((r >> 2) & 3): the 16-byte MFMA
 // operand reads of 16 consecutive rows then cover all 64 LDS banks exactly once.  The copy engine
 // writes lane l of a wave instruction to bytes [16 l, 16 l + 16) behind a wave-uniform base, so the
 // swizzle is applied on the global side (the lane landing in slot s of row r fetches chunk
 // s ^ swz(r)).
 //
-// mxfp8 scales ride along: per stage, lane l of wave v copies the 4-scale dword of row 64 v + l
-// (waves 0-3: token rows, from the row-major activation scales; waves 4-7: weight rows, from the
-// blocked weight scales) that covers the 128-wide K tile the slab lies in.
+// mxfp8 scales ride along: the 4-scale dword (128 K) of every row of the tile is copied with each
+// slab into the stage's scale region, 4 bytes per lane.
 //
 // All copies are issued as inline assembly: the compiler cannot tell the stage being read from
 // the stages being filled and would otherwise make every LDS read wait for all copies in
-// flight.  The hardware load counter (vmcnt) still counts them, in issue order; wait_pending(n)
-// lets the n most recent wave instructions stay in flight.
+// flight.  The hardware load counter (vmcnt) still counts them, per wave and in issue order; a
+// wave that issues `lps` copy instructions per stage has slab k when at most lps * (stages still
+// behind it) of its copies are pending.
 #pragma once
 #include "moe_tile.h"
 
 namespace pmoe {
 namespace ring {
 
-constexpr int kRB = 64;        // row bytes of a slab
-constexpr int kStages = 4;
-constexpr int kTokRows = 256;  // two groups of 128
-constexpr int kTokRegion = kTokRows * kRB;           // 16 KB
-constexpr int kGroupRegion = kBlockRows * kRB;       // 8 KB
-constexpr int kWRegion = kWRows * kRB;               // 16 KB
-constexpr int kScaleOff = kTokRegion + kWRegion;     // scale dwords of the 512 rows (mxfp8)
+constexpr int kRB = 64;  // row bytes of a slab
+
+template <int DT, bool SKINNY>
+struct Cfg {
+    static constexpr int kStages = SKINNY ? 8 : 4;
+    static constexpr int kTokRows = SKINNY ? 32 : 256;
+    static constexpr int kTokRegion = kTokRows * kRB;
+    static constexpr int kWRegion = kWRows * kRB;  // 16 KB
+    static constexpr int kScaleOff = kTokRegion + kWRegion;
+    static constexpr int kScaleTokRows = SKINNY ? 64 : 256;  // token scale dwords (a whole wave instruction)
+    static constexpr int kStageBytes = kScaleOff + (DT == DT_FP8 ? (kScaleTokRows + kWRows) * 4 : 0);
+    static constexpr int kRingBytes = kStages * kStageBytes;
+};
 template <int DT>
-constexpr int stage_bytes() { return kScaleOff + (DT == DT_FP8 ? 512 * 4 : 0); }
-template <int DT>
-constexpr int loads_per_stage() { return DT == DT_FP8 ? 5 : 4; }  // wave instructions per stage
+constexpr int ring_bytes() {
+    return Cfg<DT, true>::kRingBytes > Cfg<DT, false>::kRingBytes ? Cfg<DT, true>::kRingBytes : Cfg<DT, false>::kRingBytes;
+}
+constexpr int kGroupRegion = kBlockRows * kRB;  // one group's 128 token rows in the wide layout
 
 __device__ __forceinline__ int swz64(int row) { return (row >> 2) & 3; }
 
@@ -52,35 +63,49 @@ __device__ __forceinline__ void copy16(const char *base, uint32_t voff, const ch
 __device__ __forceinline__ void copy4(const char *base, uint32_t voff, const char *lds_dst) {
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr(lds_dst)) : "memory");
 }
-// Waits until at most N of this wave's copies are in flight and its LDS reads have returned, then
-// joins the workgroup barrier.
 template <int N>
 __device__ __forceinline__ void wait_and_barrier() {
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
 }
+// Waits until at most `n` (wave-uniform, <= 28) of this wave's copies are in flight and its LDS
+// reads have returned, then joins the workgroup barrier.  The wait count is an immediate of the
+// instruction, hence the switch.
+__device__ __forceinline__ void wait_and_barrier_dyn(int n) {
+    switch (n) {
+#define PMOE_WB(k) case k: wait_and_barrier<k>(); break;
+        PMOE_WB(1) PMOE_WB(2) PMOE_WB(3) PMOE_WB(4) PMOE_WB(5) PMOE_WB(6) PMOE_WB(7) PMOE_WB(8) PMOE_WB(9)
+        PMOE_WB(10) PMOE_WB(11) PMOE_WB(12) PMOE_WB(13) PMOE_WB(14) PMOE_WB(15) PMOE_WB(16) PMOE_WB(17)
+        PMOE_WB(18) PMOE_WB(19) PMOE_WB(20) PMOE_WB(21) PMOE_WB(22) PMOE_WB(23) PMOE_WB(24) PMOE_WB(25)
+        PMOE_WB(26) PMOE_WB(27) PMOE_WB(28)
+#undef PMOE_WB
+        default: wait_and_barrier<0>(); break;
+    }
+}
 
-// Per-thread description of the copies of one stage.  Thread t moves slot (t & 3) of row
-// (t >> 2) of each 128-row pass: pass 0 / 1 of the token rows are the two groups, pass 0 / 1 of the
-// weight rows are the two 128-row halves of the tile.
+// Per-thread description of the copies of one stage.  Every wave copies its 16 rows of both
+// 128-row halves of the weight tile.  Token rows: up to two wave instructions (wide: the wave's 16
+// rows of each group's block, if that block has live rows there; skinny: waves 0-1 copy the 32
+// rows).  Scales: at most one 4-byte-per-lane instruction per wave.
 struct Loader {
     const char *tok_base;
     const char *w_base[2];
     uint32_t tok_off[2];
     uint32_t w_off;
-    const char *sc_base;  // wave-uniform: activation scales (waves 0-3) or weight scales (4-7)
+    const char *sc_base;  // wave-uniform: activation scales or weight scales
     uint32_t sc_off;      // this lane's row in them
     uint32_t sc_step;     // bytes between consecutive 128-wide K tiles: 4 (row major) or 512 (blocked)
-    int wave_off;         // this wave's 16 rows inside a pass
-    int wave_sc_off;      // this wave's 64 scale dwords inside a stage
+    int tok_dst[2];       // LDS offset inside a stage of this wave's token rows; -1: nothing to copy
+    int w_dst[2];         // LDS offsets of this wave's weight rows
+    int sc_dst;           // LDS offset of this wave's scale dwords; -1: none
+    int lps;              // copy instructions this wave issues per stage
 
-    template <int DT>
     __device__ __forceinline__ void issue(char *stage, int slab) const {
         const uint32_t koff = (uint32_t)slab * kRB;
-        copy16(tok_base, tok_off[0] + koff, stage + wave_off);
-        copy16(tok_base, tok_off[1] + koff, stage + kGroupRegion + wave_off);
-        copy16(w_base[0], w_off + koff, stage + kTokRegion + wave_off);
-        copy16(w_base[1], w_off + koff, stage + kTokRegion + kWRegion / 2 + wave_off);
-        if constexpr (DT == DT_FP8) copy4(sc_base, sc_off + (uint32_t)(slab >> 1) * sc_step, stage + kScaleOff + wave_sc_off);
+        if (tok_dst[0] >= 0) copy16(tok_base, tok_off[0] + koff, stage + tok_dst[0]);
+        if (tok_dst[1] >= 0) copy16(tok_base, tok_off[1] + koff, stage + tok_dst[1]);
+        copy16(w_base[0], w_off + koff, stage + w_dst[0]);
+        copy16(w_base[1], w_off + koff, stage + w_dst[1]);
+        if (sc_dst >= 0) copy4(sc_base, sc_off + (uint32_t)(slab >> 1) * sc_step, stage + sc_dst);
     }
 };
 
@@ -154,25 +179,32 @@ __device__ __forceinline__ void mma_fp8_slab(f32x16 (&acc)[2][4], const char *to
         }
 }
 
-// K loop.  COMPUTE = false is the loop of the waves of a group without live rows: they only
-// issue their share of the copies and join the barriers.
+// K loop.  COMPUTE = false is the loop of the waves without matrix work (a group without live
+// rows; waves 4-7 of a skinny tile): they only issue their share of the copies and join the
+// barriers.  `tok_region` = byte offset of this wave's token rows inside a stage.
 //
-// The slabs are visited in rotated order, starting at slab `start` (even): with row pitches that
-// are multiples of 4 KB every row of a slab maps to the same memory channel, and workgroups that
-// all walk K from 0 would queue on one channel at a time; giving concurrent workgroups different
-// starting points spreads them over the channels.  The sum over K does not depend on the order.
-template <int DT, int NTF, bool TRANSPOSED, bool COMPUTE>
+// The slabs are visited in rotated order, starting at slab `start` (even): workgroups that run
+// side by side and share rows then ask for different cache lines at any one time instead of
+// queueing on the same ones.  The sum over K does not depend on the order.
+//
+// FULL: every wave of the workgroup issues the maximum number of copies per stage (a wide tile whose
+// two blocks are completely live), so the wait counts are compile-time constants; otherwise they
+// are computed per wave and dispatched through a switch.
+template <int DT, bool SKINNY, int NTF, bool TRANSPOSED, bool COMPUTE, bool FULL>
 __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader &ld, char *lds, int n_slabs,
-                                          const int (&wrow)[2], int lane, int grp, int start) {
-    constexpr int SB = stage_bytes<DT>();
-    constexpr int LPS = loads_per_stage<DT>();
+                                          const int (&wrow)[2], int lane, int tok_region, int start) {
+    using C = Cfg<DT, SKINNY>;
+    constexpr int SB = C::kStageBytes;
+    constexpr int NS = C::kStages;
+    constexpr int LPS_FULL = DT == DT_FP8 ? 5 : 4;
+    static_assert(!FULL || (!SKINNY && NS == 4), "constant wait counts are written for the 4-stage ring");
     auto rot = [&](int s) {
         s += start;
         return s >= n_slabs ? s - n_slabs : s;
     };
 #pragma unroll
-    for (int s = 0; s < kStages - 1; ++s)
-        if (s < n_slabs) ld.template issue<DT>(lds + s * SB, rot(s));
+    for (int s = 0; s < NS - 1; ++s)
+        if (s < n_slabs) ld.issue(lds + s * SB, rot(s));
     FragsBf16 fx, fy;  // fy carries the held-back sub-step across the barrier
     if constexpr (DT == DT_BF16 && COMPUTE) {
 #pragma unroll
@@ -184,17 +216,22 @@ __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader &ld,
 #pragma unroll
             for (int i = 0; i < 8; ++i) fy.b[t][i] = (__bf16)0.0f;
     }
+    const int lps = ld.lps;
     for (int kt = 0; kt < n_slabs; ++kt) {
-        // slab kt has landed once at most the copies of the (up to two) later slabs are in flight
-        if (kt + 2 < n_slabs) wait_and_barrier<2 * LPS>();
-        else if (kt + 1 < n_slabs) wait_and_barrier<LPS>();
-        else wait_and_barrier<0>();
+        // slab kt has landed once at most the copies of the later slabs (up to NS - 2) are pending
+        if constexpr (FULL) {
+            if (kt + 2 < n_slabs) wait_and_barrier<2 * LPS_FULL>();
+            else if (kt + 1 < n_slabs) wait_and_barrier<LPS_FULL>();
+            else wait_and_barrier<0>();
+        } else {
+            wait_and_barrier_dyn(lps * min(NS - 2, n_slabs - 1 - kt));
+        }
         // the stage consumed in the previous iteration is free: everybody is past the barrier
-        if (kt + kStages - 1 < n_slabs) ld.template issue<DT>(lds + ((kt + kStages - 1) & (kStages - 1)) * SB, rot(kt + kStages - 1));
+        if (kt + NS - 1 < n_slabs) ld.issue(lds + ((kt + NS - 1) & (NS - 1)) * SB, rot(kt + NS - 1));
         if constexpr (COMPUTE) {
-            const char *cur = lds + (kt & (kStages - 1)) * SB;
-            const char *tok = cur + grp * kGroupRegion;
-            const char *wgt = cur + kTokRegion;
+            const char *cur = lds + (kt & (NS - 1)) * SB;
+            const char *tok = cur + tok_region;
+            const char *wgt = cur + C::kTokRegion;
             if constexpr (DT == DT_BF16) {
                 // software pipeline across the barrier: the second K sub-step of a slab is held back
                 // and issued behind the first fragment reads of the next slab
@@ -216,9 +253,10 @@ __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader &ld,
                     }
                 }
             } else {
-                const uint32_t *sc = reinterpret_cast<const uint32_t *>(cur + kScaleOff);
-                mma_fp8_slab<NTF, TRANSPOSED>(acc, tok, wgt, sc + grp * kBlockRows, sc + kTokRows, wrow, lane,
-                                              8 * (2 * (kt & 1) + (lane >> 5)));  // start is even: parity of kt = parity of the slab
+                const uint32_t *sc = reinterpret_cast<const uint32_t *>(cur + C::kScaleOff);
+                // start is even: the parity of kt is the parity of the slab inside its 128-wide K tile
+                mma_fp8_slab<NTF, TRANSPOSED>(acc, tok, wgt, sc + tok_region / kRB, sc + C::kScaleTokRows, wrow, lane,
+                                              8 * (2 * (kt & 1) + (lane >> 5)));
             }
         }
     }

@@ -15,6 +15,7 @@
 #include <algorithm>
 
 #include "moe_ring.h"
+#include "moe_ring128.h"
 #include "moe_tile.h"
 #include "pmoe_common.h"
 
@@ -320,6 +321,7 @@ __device__ __forceinline__ void setup_ring_loader(ring::Loader &ld, int tid, uin
         }
     }
     ld.lps = 2 + (ld.tok_dst[0] >= 0) + (ld.tok_dst[1] >= 0) + (ld.sc_dst >= 0);
+    ld.make_uniform();
 }
 
 // First slab of this workgroup's walk over K: workgroups that run side by side on an XCD (consecutive
@@ -379,11 +381,62 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
     if (active) store_act_tile<DT>(a, tile, sc_tile, (int64_t)(first + grp) * kBlockRows, h0, my_ntf, gt);
 }
 
+// LDS plan of the split kernels.  bf16: the 160 KB ring of the wide engine is all the LDS there is;
+// the row table sits in the tail of its last unit, which the ring first fills after the barrier
+// that opens slab 0, when the loaders hold everything they need of it in registers (the skinny
+// ring is shorter and never reaches it).  mxfp8: ring, row table, activation scales side by side.
+template <int DT>
+struct SplitLds {
+    static constexpr int kRowInfoBytes = 2304;  // >= sizeof(RowInfo<2>)
+    static constexpr int kRing = DT == DT_BF16 ? ring128::kRingBytes : ring::ring_bytes<DT>();
+    static constexpr int kRowInfoOff = DT == DT_BF16 ? kRing - kRowInfoBytes : kRing;
+    static constexpr int kActScaleOff = kRowInfoOff + kRowInfoBytes;  // mxfp8 only
+    static constexpr int kTotal = DT == DT_BF16 ? kRing : kActScaleOff + kBlockRows * 2 * 4;
+    static_assert(sizeof(RowInfo<2>) <= kRowInfoBytes, "row table does not fit its slot");
+    static_assert(DT != DT_BF16 || ring::Cfg<DT_BF16, true>::kRingBytes <= kRowInfoOff, "skinny ring reaches the row table");
+};
+
+// First slab of a wide bf16 tile's walk over K: 8 phases, one 128-byte slab apart.
+__device__ __forceinline__ int slab_rotation128(int n_slabs) { return (int)((blockIdx.x >> 3) & 7) % n_slabs; }
+
+// Up kernel tile on the 128-byte ring (bf16, two blocks or one block with more than 32 live rows).
+template <int NTF>
+__device__ __forceinline__ void up_tile_wide_bf16(const MoeArgs &a, int first, int ht, int e, RowInfo<2> &ri, char *lds) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
+    const int K = a.K, H = a.H, N = a.N;
+    const int h0 = ht * 128;
+    const int ntf0 = __builtin_amdgcn_readfirstlane((ri.nvalid[0] + 31) >> 5);
+    const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
+    const int my_ntf = grp ? ntf1 : ntf0;
+    const bool active = my_ntf > 0;
+
+    const uint32_t row_bytes = (uint32_t)K * 2u;
+    const char *w_gate = a.w1 + ((int64_t)e * N + h0) * K * 2;
+    ring128::Loader ld;
+    ld.setup(tid, a.x, w_gate, w_gate + (int64_t)H * K * 2, row_bytes, ntf0, ntf1,
+             [&](int row) { return (uint32_t)max(ri.tok[row], 0) * row_bytes; });  // dead rows read token 0
+
+    const int wrow[2] = {32 * w4, 128 + 32 * w4};
+    f32x16 acc[2][4];
+    zero_acc(acc);
+    const int n_slabs = (int)(row_bytes / ring128::kRB);
+    const int start = slab_rotation128(n_slabs);
+    const int tok_region = grp * ring128::kGroupRegion;
+    if (active) ring128::main_loop<NTF, true, true>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
+    else ring128::main_loop<NTF, true, false>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
+
+    char *tile = lds + grp * (kBlockRows * kActPitchBf16);
+    if (active) swiglu_epilogue<DT_BF16, false, NTF>(acc, tile, nullptr, w4, lane);
+    __syncthreads();
+    if (active) store_act_tile<DT_BF16>(a, tile, nullptr, (int64_t)(first + grp) * kBlockRows, h0, my_ntf, gt);
+}
+
 template <int DT>
 __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
-    __shared__ __attribute__((aligned(1024))) char lds[ring::ring_bytes<DT>()];
-    __shared__ uint32_t act_sc_lds[kBlockRows * 2];
-    __shared__ RowInfo<2> ri;
+    using L = SplitLds<DT>;
+    __shared__ __attribute__((aligned(1024))) char lds[L::kTotal];
+    RowInfo<2> &ri = *reinterpret_cast<RowInfo<2> *>(lds + L::kRowInfoOff);
     int first, nb, ht;
     if (!resolve_tile<2>(a, first, nb, ht)) return;
     if (first * kBlockRows >= a.ntpp[0]) return;
@@ -391,12 +444,21 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
     if (ntf == 0) return;
     const int e = a.expert_ids[first];
     if (e < 0 || e >= a.E) return;
-    const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-    if (ntf == 1 && ri.nvalid[1] == 0) up_tile_ring<DT, true, 1, false>(a, first, ht, e, ri, lds, act_sc_lds);
-    else if (ntf == 1) up_tile_ring<DT, false, 1, false>(a, first, ht, e, ri, lds, act_sc_lds);
-    else if (ntf == 2) up_tile_ring<DT, false, 2, false>(a, first, ht, e, ri, lds, act_sc_lds);
-    else if (full) up_tile_ring<DT, false, 4, true>(a, first, ht, e, ri, lds, act_sc_lds);
-    else up_tile_ring<DT, false, 4, false>(a, first, ht, e, ri, lds, act_sc_lds);
+    const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
+    if constexpr (DT == DT_BF16) {
+        if (skinny) up_tile_ring<DT, true, 1, false>(a, first, ht, e, ri, lds, nullptr);
+        else if (ntf == 1) up_tile_wide_bf16<1>(a, first, ht, e, ri, lds);
+        else if (ntf == 2) up_tile_wide_bf16<2>(a, first, ht, e, ri, lds);
+        else up_tile_wide_bf16<4>(a, first, ht, e, ri, lds);
+    } else {
+        uint32_t *act_sc_lds = reinterpret_cast<uint32_t *>(lds + L::kActScaleOff);
+        const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
+        if (skinny) up_tile_ring<DT, true, 1, false>(a, first, ht, e, ri, lds, act_sc_lds);
+        else if (ntf == 1) up_tile_ring<DT, false, 1, false>(a, first, ht, e, ri, lds, act_sc_lds);
+        else if (ntf == 2) up_tile_ring<DT, false, 2, false>(a, first, ht, e, ri, lds, act_sc_lds);
+        else if (full) up_tile_ring<DT, false, 4, true>(a, first, ht, e, ri, lds, act_sc_lds);
+        else up_tile_ring<DT, false, 4, false>(a, first, ht, e, ri, lds, act_sc_lds);
+    }
 }
 
 // Down kernel of the split pipeline: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
@@ -439,10 +501,46 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     }
 }
 
+// Down kernel tile on the 128-byte ring (bf16).  The ring overwrites the row table; every thread
+// carries one of its 512 words through the K loop in a register and puts it back for the scatter.
+template <int NTF>
+__device__ __forceinline__ void down_tile_wide_bf16(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, char *lds) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int grp = wave >> 2, w4 = wave & 3;
+    const int K = a.K, H = a.H;
+    const int k0 = kt * kWRows;
+    const int64_t row0 = (int64_t)first * kBlockRows;
+    const int ntf0 = __builtin_amdgcn_readfirstlane((ri.nvalid[0] + 31) >> 5);
+    const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
+    const bool active = (grp ? ntf1 : ntf0) > 0;
+    const int kept = tid < 2 * kBlockRows ? ri.tok[tid] : __float_as_int(ri.wt[tid - 2 * kBlockRows]);
+
+    const uint32_t row_bytes = (uint32_t)H * 2u;
+    const char *w_lo = a.w2 + ((int64_t)e * K + k0) * H * 2;
+    const char *w_hi = (k0 + 128 < K) ? w_lo + (int64_t)128 * H * 2 : w_lo;
+    ring128::Loader ld;
+    ld.setup(tid, a.act + row0 * H * 2, w_lo, w_hi, row_bytes, ntf0, ntf1,
+             [&](int row) { return (uint32_t)row * row_bytes; });
+
+    const int wrow[2] = {64 * w4, 64 * w4 + 32};
+    f32x16 acc[2][4];
+    zero_acc(acc);
+    const int n_slabs = (int)(row_bytes / ring128::kRB);
+    const int start = slab_rotation128(n_slabs);
+    const int tok_region = grp * ring128::kGroupRegion;
+    if (active) ring128::main_loop<NTF, false, true>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
+    else ring128::main_loop<NTF, false, false>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
+    if (tid < 2 * kBlockRows) ri.tok[tid] = kept;
+    else ri.wt[tid - 2 * kBlockRows] = __int_as_float(kept);
+    __syncthreads();
+    if (active) scatter_add<NTF>(acc, ri.tok + grp * kBlockRows, ri.wt + grp * kBlockRows, a.accum, K, k0 + 64 * w4, lane);
+}
+
 template <int DT>
 __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
-    __shared__ __attribute__((aligned(1024))) char lds[ring::ring_bytes<DT>()];
-    __shared__ RowInfo<2> ri;
+    using L = SplitLds<DT>;
+    __shared__ __attribute__((aligned(1024))) char lds[L::kTotal];
+    RowInfo<2> &ri = *reinterpret_cast<RowInfo<2> *>(lds + L::kRowInfoOff);
     int first, nb, kt;
     if (!resolve_tile<2>(a, first, nb, kt)) return;
     if (first * kBlockRows >= a.ntpp[0]) return;
@@ -450,12 +548,20 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
     if (ntf == 0) return;
     const int e = a.expert_ids[first];
     if (e < 0 || e >= a.E) return;
-    const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-    if (ntf == 1 && ri.nvalid[1] == 0) down_tile_ring<DT, true, 1, false>(a, first, kt, e, ri, lds);
-    else if (ntf == 1) down_tile_ring<DT, false, 1, false>(a, first, kt, e, ri, lds);
-    else if (ntf == 2) down_tile_ring<DT, false, 2, false>(a, first, kt, e, ri, lds);
-    else if (full) down_tile_ring<DT, false, 4, true>(a, first, kt, e, ri, lds);
-    else down_tile_ring<DT, false, 4, false>(a, first, kt, e, ri, lds);
+    const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
+    if constexpr (DT == DT_BF16) {
+        if (skinny) down_tile_ring<DT, true, 1, false>(a, first, kt, e, ri, lds);
+        else if (ntf == 1) down_tile_wide_bf16<1>(a, first, kt, e, ri, lds);
+        else if (ntf == 2) down_tile_wide_bf16<2>(a, first, kt, e, ri, lds);
+        else down_tile_wide_bf16<4>(a, first, kt, e, ri, lds);
+    } else {
+        const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
+        if (skinny) down_tile_ring<DT, true, 1, false>(a, first, kt, e, ri, lds);
+        else if (ntf == 1) down_tile_ring<DT, false, 1, false>(a, first, kt, e, ri, lds);
+        else if (ntf == 2) down_tile_ring<DT, false, 2, false>(a, first, kt, e, ri, lds);
+        else if (full) down_tile_ring<DT, false, 4, true>(a, first, kt, e, ri, lds);
+        else down_tile_ring<DT, false, 4, false>(a, first, kt, e, ri, lds);
+    }
 }
 
 // ==========================================================================================

@@ -63,6 +63,13 @@ __device__ __forceinline__ void copy16(const char *base, uint32_t voff, const ch
 __device__ __forceinline__ void copy4(const char *base, uint32_t voff, const char *lds_dst) {
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr(lds_dst)) : "memory");
 }
+// A wave-uniform pointer, read through lane 0 so that the compiler keeps it in scalar registers.
+__device__ __forceinline__ const char *uniform_ptr(const char *p) {
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const char *)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
 template <int N>
 __device__ __forceinline__ void wait_and_barrier() {
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
@@ -98,6 +105,14 @@ struct Loader {
     int w_dst[2];         // LDS offsets of this wave's weight rows
     int sc_dst;           // LDS offset of this wave's scale dwords; -1: none
     int lps;              // copy instructions this wave issues per stage
+
+    // The base pointers feed scalar operands of the copy instructions: pin them to scalar registers.
+    __device__ __forceinline__ void make_uniform() {
+        tok_base = uniform_ptr(tok_base);
+        w_base[0] = uniform_ptr(w_base[0]);
+        w_base[1] = uniform_ptr(w_base[1]);
+        sc_base = uniform_ptr(sc_base);
+    }
 
     __device__ __forceinline__ void issue(char *stage, int slab) const {
         const uint32_t koff = (uint32_t)slab * kRB;

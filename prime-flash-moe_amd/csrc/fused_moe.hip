@@ -186,8 +186,8 @@ __device__ __forceinline__ void swiglu_epilogue(const f32x16 (&acc)[2][4], char 
                 for (int g = 0; g < 4; ++g) {
                     const int hl = 32 * w4 + 8 * g + 4 * half;  // tile-local activation column
                     uint2 pk;
-                    pk.x = f32_to_bf16_bits(v[4 * g]) | (f32_to_bf16_bits(v[4 * g + 1]) << 16);
-                    pk.y = f32_to_bf16_bits(v[4 * g + 2]) | (f32_to_bf16_bits(v[4 * g + 3]) << 16);
+                    pk.x = pack2_bf16(v[4 * g], v[4 * g + 1]);
+                    pk.y = pack2_bf16(v[4 * g + 2], v[4 * g + 3]);
                     char *dst;
                     if constexpr (OPERAND) {
                         const int byte = (hl & 63) * 2;
@@ -862,7 +862,7 @@ __global__ __launch_bounds__(256) void finalize_kernel(const float4 *acc, uint4 
             }
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) o[j] = f32_to_bf16_bits(v[2 * j]) | (f32_to_bf16_bits(v[2 * j + 1]) << 16);
+        for (int j = 0; j < 4; ++j) o[j] = pack2_bf16(v[2 * j], v[2 * j + 1]);
         out[i] = make_uint4(o[0], o[1], o[2], o[3]);
     }
 }

@@ -60,16 +60,25 @@ struct Loader {
         tok_base = ring::uniform_ptr(tok);
         w_base = ring::uniform_ptr(wave < 4 ? w_half0 : w_half1);
     }
-    __device__ __forceinline__ void issue_w(char *unit, int slab) const {
+    // Copies i0 and i0 + 1 (of 4) of this wave's share of a weight / token unit.
+    __device__ __forceinline__ void issue_w2(char *unit, int slab, int i0) const {
         const uint32_t koff = (uint32_t)slab * kRB;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ring::copy16(w_base, w_off[i] + koff, unit + dst + i * 8 * kRB);
+        for (int i = i0; i < i0 + 2; ++i) ring::copy16(w_base, w_off[i] + koff, unit + dst + i * 8 * kRB);
     }
-    __device__ __forceinline__ void issue_t(char *unit, int slab) const {
+    __device__ __forceinline__ void issue_t2(char *unit, int slab, int i0) const {
         if (!tok_live) return;
         const uint32_t koff = (uint32_t)slab * kRB;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ring::copy16(tok_base, tok_off[i] + koff, unit + dst + i * 8 * kRB);
+        for (int i = i0; i < i0 + 2; ++i) ring::copy16(tok_base, tok_off[i] + koff, unit + dst + i * 8 * kRB);
+    }
+    __device__ __forceinline__ void issue_w(char *unit, int slab) const {
+        issue_w2(unit, slab, 0);
+        issue_w2(unit, slab, 2);
+    }
+    __device__ __forceinline__ void issue_t(char *unit, int slab) const {
+        issue_t2(unit, slab, 0);
+        issue_t2(unit, slab, 2);
     }
 };
 
@@ -132,24 +141,36 @@ __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader &ld,
     for (int kt = 0; kt < n_slabs; ++kt) {
         if (kt + 1 < n_slabs) ring::wait_and_barrier<4>();
         else ring::wait_and_barrier<0>();
-        // everybody is past the barrier: the buffers of slab kt - 1 (bw + 3, bw + 4) are free
-        if (kt + 1 < n_slabs) ld.issue_t(lds + next(bw, 3) * kUnitBytes, rot(kt + 1));
-        if (kt + 2 < n_slabs) ld.issue_w(lds + next(bw, 4) * kUnitBytes, rot(kt + 2));
+        // Everybody is past the barrier: the buffers of slab kt - 1 (bw + 3, bw + 4) are free.  Their
+        // refill (token unit kt + 1, then weight unit kt + 2) is spread over the slab, two copies per
+        // quarter, so that the copy instructions of the eight waves reach the memory pipeline at the
+        // rate it retires them instead of queueing in front of every wave's matrix instructions.
+        char *t_unit = lds + next(bw, 3) * kUnitBytes;
+        char *w_unit = lds + next(bw, 4) * kUnitBytes;
+        const bool more_t = kt + 1 < n_slabs, more_w = kt + 2 < n_slabs;
+        const int t_slab = rot(kt + 1), w_slab = rot(kt + 2);
         if constexpr (COMPUTE) {
             const char *wgt = lds + bw * kUnitBytes;
             const char *tok = lds + next(bw, 1) * kUnitBytes + tok_region;
+            if (more_t) ld.issue_t2(t_unit, t_slab, 0);
             fetch<NTF>(fx, tok, wgt, wrow, lane, 0);
             ring::mma_bf16<NTF, TRANSPOSED>(acc, fy);
             interleave_pair<NTF>();
+            if (more_t) ld.issue_t2(t_unit, t_slab, 2);
             fetch<NTF>(fy, tok, wgt, wrow, lane, 1);
             ring::mma_bf16<NTF, TRANSPOSED>(acc, fx);
             interleave_pair<NTF>();
+            if (more_w) ld.issue_w2(w_unit, w_slab, 0);
             fetch<NTF>(fx, tok, wgt, wrow, lane, 2);
             ring::mma_bf16<NTF, TRANSPOSED>(acc, fy);
             interleave_pair<NTF>();
+            if (more_w) ld.issue_w2(w_unit, w_slab, 2);
             fetch<NTF>(fy, tok, wgt, wrow, lane, 3);
             ring::mma_bf16<NTF, TRANSPOSED>(acc, fx);
             interleave_pair<NTF>();
+        } else {
+            if (more_t) ld.issue_t(t_unit, t_slab);
+            if (more_w) ld.issue_w(w_unit, w_slab);
         }
         bw = next(bw, 2);
     }

@@ -61,8 +61,17 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
 }
 
+// Two fp32 -> one dword of two bf16 (round to nearest even), the hardware conversion of gfx950.
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const bf16x2 v = __builtin_convertvector(f32x2{lo, hi}, bf16x2);
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+// silu(gate) * up with the hardware exponential and reciprocal (about 1 ulp each, far inside bf16).
 __device__ __forceinline__ float swiglu(float gate, float up) {
-    return up * gate / (1.0f + __expf(-gate));
+    return up * gate * __builtin_amdgcn_rcpf(1.0f + __expf(-gate));
 }
 
 // OCP-MX shared scale of a 32-block with absolute maximum `amax`:

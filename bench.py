@@ -156,7 +156,7 @@ def run_config(cfg, split, steps, warmup, device, with_cpu, log):
     sec = time_steps(step, steps, warmup)
     ev_mean, ev_med = time_events(step, steps)
     t_up = phase_time(step, PHASE_UP, steps)
-    t_down = phase_time(step, PHASE_DOWN, steps) if split else 0.0
+    t_down = phase_time(step, PHASE_DOWN, steps)
     step()
     torch.cuda.synchronize()
     P = cfg.T * cfg.top_k
@@ -239,7 +239,7 @@ def main():
                     "peak": PEAK_TFLOPS[cfg.dtype], "unit": "TFLOP/s",
                     "kernel": "moe_up_kernel (gate/up GEMM + SwiGLU)", "launch_us": r["t_up"] * 1e6}
     roofline["frac"] = roofline["achieved"] / roofline["peak"]
-    roofline["traffic"] = MEASURED_TRAFFIC.get((cfg.name, int(bool(args.split))))
+    roofline["traffic"] = MEASURED_TRAFFIC.get((cfg.name, 1))  # the kernels do not depend on --split
     line = {
         "metric": "Fused-MoE TFLOP/s & % MFMA peak (bf16/mxfp8); decode-shape HBM GB/s",
         "value": r["weight_gbs"] if memory_bound else r["tflops"],

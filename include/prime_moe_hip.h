@@ -55,6 +55,8 @@ int pmoe_moe_align(const int32_t *topk_ids, int32_t *sorted_token_ids, int32_t *
 /*
  * Workspace (bytes) the fused calls below need for a problem of this size.  The
  * caller allocates it on the device (any 256-byte aligned buffer) and passes it in.
+ * The size does not depend on `split` (both values run the same kernels); the argument
+ * is kept so that the query takes what the call takes.
  */
 size_t pmoe_fused_moe_bf16_workspace_bytes(int M, int K, int N, int num_experts, int sorted_num,
                                            int split);
@@ -70,6 +72,8 @@ size_t pmoe_fused_moe_mxfp8_workspace_bytes(int M, int K, int N, int num_experts
  *               topk_weights[p] * W2[e] . swiglu(W1[e] . x[t]),  e = expert_idxs[s/block_m].
  * split != 0: `out` is overwritten (the reference zeroes it itself and adds).
  * split == 0: the result is added to `out`; the caller pre-zeroes it.
+ * Either way the work is done by the same up and down kernels with the activation in the
+ * workspace; `split` selects only how the last kernel treats `out`.
  * block_n / warp_n / stages are validated exactly as the reference does and then
  * ignored (they size Blackwell thread blocks and smem rings); block_m must be 128,
  * bpc == cpc == 1, K % 128 == 0, N % 256 == 0.
@@ -114,8 +118,8 @@ int pmoe_quantize_mx(const void *src_bf16, void *q, void *scales, int64_t rows, 
  * with events around the call.  Results are only meaningful with PMOE_PHASE_ALL (the default).
  */
 #define PMOE_PHASE_ZERO 1     /* clear the fp32 accumulator */
-#define PMOE_PHASE_UP 2       /* gate/up GEMM + SwiGLU (the whole fused kernel when split == 0) */
-#define PMOE_PHASE_DOWN 4     /* down GEMM of the split pipeline */
+#define PMOE_PHASE_UP 2       /* gate/up GEMM + SwiGLU */
+#define PMOE_PHASE_DOWN 4     /* down GEMM + routing-weight reduction */
 #define PMOE_PHASE_FINALIZE 8 /* accumulator -> bf16 `out` */
 #define PMOE_PHASE_ALL 15
 void pmoe_set_phase_mask(int mask);

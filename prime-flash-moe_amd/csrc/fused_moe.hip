@@ -4,13 +4,14 @@
 // Replaces the launchers and kernels of the reference's
 // prime_moe/csrc/kernels/fused_moe_bf16_kernel.cu:21-733 and fused_moe_mxfp8_kernel.cu:56-866.
 //
-// Pipelines
-//   split != 0 : zero(accum) -> up kernel (act tile -> workspace) -> down kernel (fp32 atomics
-//                into accum, one addend per routed pair) -> finalize (out = bf16(accum)).
-//   split == 0 : zero(accum) -> fused kernel: up phase leaves the 128x128 activation tile in LDS
-//                in MFMA operand layout, the down phase streams W2[e][:, h-slice] against it and
-//                adds every 128x256 partial product into accum (split-K over H/128 workgroups)
-//                -> finalize (out += bf16(accum)).
+// Pipeline of one call (all on the caller's stream):
+//   prologue (zero the fp32 accumulator, pair blocks into row tiles, build the two work lists)
+//   -> up kernel (gate/up GEMM + SwiGLU, activation tile -> workspace)
+//   -> down kernel (fp32 atomics into the accumulator, one addend per routed pair)
+//   -> finalize: split != 0: out = bf16(accum); split == 0: out = bf16(float(out) + accum), the
+//      reference's accumulate-into-out contract of its single-kernel path.
+// Both values of `split` run the same kernels: on this hardware the two-kernel pipeline is the faster
+// one at every shape, so `split` only selects what finalize does with `out`.
 // The top-k reduction is exact in fp32 up to summation order; `out` is rounded to bf16 once.
 #include <algorithm>
 
@@ -46,44 +47,21 @@ struct MoeArgs {
 constexpr int kActPitchBf16 = 272;  // 128 bf16 + 16 B pad: 16-byte aligned rows, 2-way conflicts at most
 constexpr int kActPitchFp8 = 144;   // 128 e4m3 + 16 B pad
 
-// Workgroup id -> (row tile, weight tile), using the live tile count read on the device.
+// Workgroup id -> (first block, blocks, weight tile), using the live tile count read on the device.
 // Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; ids are regrouped so that
-// one XCD runs a contiguous range of logical ids.  The two-group kernels then look their tile up in
-// the work list the prologue built (expert-major order, see moe_prologue_kernel); the single-group
-// fused kernel walks [group of 8 weight tiles][row blocks][weight tile in group].
-template <int NG>
+// one XCD runs a contiguous range of logical ids, which index the work list the prologue built.
 __device__ __forceinline__ bool resolve_tile(const MoeArgs &a, int &first, int &nb, int &wt) {
-    int n_row_tiles;
-    if constexpr (NG == 2) n_row_tiles = min(a.n_tiles[0], a.n_blocks);
-    else n_row_tiles = min((a.ntpp[0] + kBlockRows - 1) / kBlockRows, a.n_blocks);
+    const int n_row_tiles = min(a.n_tiles[0], a.n_blocks);
     const int G = n_row_tiles * a.n_wtiles;
     const int per_xcd = (G + 7) >> 3;
     const int idx = (int)(blockIdx.x >> 3);
     if (idx >= per_xcd) return false;
     const int logical = (int)(blockIdx.x & 7) * per_xcd + idx;
     if (logical >= G) return false;
-    if constexpr (NG == 2) {
-        const int2 w = a.work[logical];
-        first = w.x & 0x0fffffff;
-        nb = w.x >> 28;
-        wt = w.y;
-    } else {
-        constexpr int GW = 8;
-        const int full = a.n_wtiles / GW * GW;
-        const int per_group = n_row_tiles * GW;
-        const int g = logical / per_group;
-        if (g * GW < full) {
-            const int rem = logical - g * per_group;
-            first = rem / GW;
-            wt = g * GW + rem % GW;
-        } else {
-            const int tw = a.n_wtiles - full;
-            const int rem = logical - (full / GW) * per_group;
-            first = rem / tw;
-            wt = full + rem % tw;
-        }
-        nb = 1;
-    }
+    const int2 w = a.work[logical];
+    first = w.x & 0x0fffffff;
+    nb = w.x >> 28;
+    wt = w.y;
     return true;
 }
 
@@ -165,12 +143,11 @@ __device__ __forceinline__ void scatter_add(const f32x16 (&acc)[2][4], const int
 // SwiGLU epilogue of the up GEMM, in registers: the 2H-wide gate/up tensor never leaves the chip.
 // acc[0] holds gate rows, acc[1] the matching up rows (weight rows on the MFMA M side: register i
 // of lane l = activation column 32 w4 + 8(i/4) + 4(l/32) + i%4 of token row 32 t + l%32).  The
-// 128 x 128 activation tile of the group is written to `tile`:
-//   OPERAND = false: row pitch kActPitch*, for the coalesced copy to the workspace;
-//   OPERAND = true : in the 128-byte-slab MFMA operand layout of the fused kernel's down phase.
+// 128 x 128 activation tile of the group is written to `tile` with row pitch kActPitch*, for the
+// coalesced copy to the workspace.
 // mxfp8: per token row and 32 columns, amax -> e8m0 scale + e4m3 values; a lane holds 16 of the 32
 // columns of one MX block, the partner lane (l ^ 32) the others.
-template <int DT, bool OPERAND, int NTF>
+template <int DT, int NTF>
 __device__ __forceinline__ void swiglu_epilogue(const f32x16 (&acc)[2][4], char *tile, uint32_t *sc_tile,
                                                 int w4, int lane) {
     const int r = lane & 31, half = lane >> 5;
@@ -188,15 +165,7 @@ __device__ __forceinline__ void swiglu_epilogue(const f32x16 (&acc)[2][4], char 
                     uint2 pk;
                     pk.x = pack2_bf16(v[4 * g], v[4 * g + 1]);
                     pk.y = pack2_bf16(v[4 * g + 2], v[4 * g + 3]);
-                    char *dst;
-                    if constexpr (OPERAND) {
-                        const int byte = (hl & 63) * 2;
-                        dst = tile + (hl >> 6) * kGroupRegion + row * kRowBytes +
-                              (((byte >> 4) ^ swz(row)) << 4) + (byte & 15);
-                    } else {
-                        dst = tile + row * kActPitchBf16 + hl * 2;
-                    }
-                    *reinterpret_cast<uint2 *>(dst) = pk;
+                    *reinterpret_cast<uint2 *>(tile + row * kActPitchBf16 + hl * 2) = pk;
                 }
             } else {
                 float amax = 0.f;
@@ -210,12 +179,7 @@ __device__ __forceinline__ void swiglu_epilogue(const f32x16 (&acc)[2][4], char 
                 for (int g = 0; g < 4; ++g) {
                     const int hl = 32 * w4 + 8 * g + 4 * half;
                     const uint32_t q = pack4_e4m3(v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3], inv);
-                    char *dst;
-                    if constexpr (OPERAND)
-                        dst = tile + row * kRowBytes + (((hl >> 4) ^ swz(row)) << 4) + (hl & 15);
-                    else
-                        dst = tile + row * kActPitchFp8 + hl;
-                    *reinterpret_cast<uint32_t *>(dst) = q;
+                    *reinterpret_cast<uint32_t *>(tile + row * kActPitchFp8 + hl) = q;
                 }
                 if (half == 0) reinterpret_cast<uint8_t *>(sc_tile)[row * 4 + w4] = (uint8_t)e8;
             }
@@ -255,42 +219,35 @@ __device__ __forceinline__ void store_act_tile(const MoeArgs &a, const char *til
 }
 
 // ==========================================================================================
-// Split pipeline, two-group kernels on the ring engine
+// Two-group kernels on the ring engines
 // ==========================================================================================
 
 // Common set-up of the ring loader.  Token rows: `tok_row_off(row)` gives the byte offset of tile
-// row `row` in `tok_base`; weight rows: the tile's two 128-row halves start at w_base[0/1] with
-// `w_pitch` bytes per row.  Scales (mxfp8): `tok_sc_off(row)` / `w_sc_off(row)` are the byte offsets
-// of the row's first 4-scale dword.  ntf0 / ntf1 = 32-row fragments with live rows in the two
-// blocks of the tile; token rows (and their scales) of dead fragments are not copied.
-template <int DT, bool SKINNY, typename TokOff, typename TokScOff, typename WScOff>
-__device__ __forceinline__ void setup_ring_loader(ring::Loader &ld, int tid, uint32_t w_pitch, int ntf0, int ntf1,
-                                                  TokOff tok_row_off, const uint8_t *tok_sc_base,
+// row `row` (0..255: block 0, then block 1) in `tok_base`; weight rows: the tile's two 128-row halves
+// start at w_base[0/1] with `w_pitch` bytes per row.  Scales (mxfp8): `tok_sc_off(row)` /
+// `w_sc_off(row)` are the byte offsets of the row's first 4-scale dword.  Only the live 32-row
+// fragments of the two blocks (ntf0, ntf1 of them) are copied; they are packed one after the other in
+// the stage (see ring::Layout).
+template <int DT, typename TokOff, typename TokScOff, typename WScOff>
+__device__ __forceinline__ void setup_ring_loader(ring::Loader &ld, const ring::Layout &lay, int tid, uint32_t w_pitch,
+                                                  int ntf0, int ntf1, TokOff tok_row_off, const uint8_t *tok_sc_base,
                                                   TokScOff tok_sc_off, const uint8_t *w_sc_base, WScOff w_sc_off) {
-    using C = ring::Cfg<DT, SKINNY>;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int prow = tid >> 2;                         // row inside a 128-row pass
     const int gchunk = (tid & 3) ^ ring::swz64(prow);  // global chunk landing in this lane's LDS slot
     ld.w_off = (uint32_t)prow * w_pitch + gchunk * 16;
-    ld.w_dst[0] = C::kTokRegion + wave * 16 * ring::kRB;
+    ld.w_dst[0] = lay.w_off + wave * 16 * ring::kRB;
     ld.w_dst[1] = ld.w_dst[0] + 128 * ring::kRB;
     ld.tok_dst[0] = ld.tok_dst[1] = -1;
     ld.tok_off[0] = ld.tok_off[1] = 0;
-    if constexpr (SKINNY) {
-        if (wave < 2) {  // 32 rows = two wave instructions
-            ld.tok_dst[0] = wave * 16 * ring::kRB;
-            ld.tok_off[0] = tok_row_off(prow) + gchunk * 16;
-        }
-    } else {
-        const int frag = wave >> 1;  // the wave's 16 rows of a block lie in this fragment
-        if (frag < ntf0) {
-            ld.tok_dst[0] = wave * 16 * ring::kRB;
-            ld.tok_off[0] = tok_row_off(prow) + gchunk * 16;
-        }
-        if (frag < ntf1) {
-            ld.tok_dst[1] = ring::kGroupRegion + wave * 16 * ring::kRB;
-            ld.tok_off[1] = tok_row_off(kBlockRows + prow) + gchunk * 16;
-        }
+    const int frag = wave >> 1;  // the wave's 16 rows of a block lie in this fragment
+    if (frag < ntf0) {
+        ld.tok_dst[0] = wave * 16 * ring::kRB;
+        ld.tok_off[0] = tok_row_off(prow) + gchunk * 16;
+    }
+    if (frag < ntf1) {
+        ld.tok_dst[1] = lay.group1_off + wave * 16 * ring::kRB;
+        ld.tok_off[1] = tok_row_off(kBlockRows + prow) + gchunk * 16;
     }
     ld.sc_base = nullptr;
     ld.sc_off = 0;
@@ -302,22 +259,15 @@ __device__ __forceinline__ void setup_ring_loader(ring::Loader &ld, int tid, uin
             ld.sc_base = reinterpret_cast<const char *>(w_sc_base);
             ld.sc_off = w_sc_off(row);
             ld.sc_step = 512u;
-            ld.sc_dst = C::kScaleOff + (C::kScaleTokRows + 64 * (wave - 4)) * 4;
-        } else if constexpr (SKINNY) {
-            if (wave == 2) {  // token rows 0..31 (the upper lanes repeat row 31 into unused dwords)
-                ld.sc_base = reinterpret_cast<const char *>(tok_sc_base);
-                ld.sc_off = tok_sc_off(min(lane, 31));
-                ld.sc_step = 4u;
-                ld.sc_dst = C::kScaleOff;
-            }
-        } else {
-            const int row = 64 * wave + lane;  // token rows: block wave / 2, fragments 2 (wave & 1), + 1
-            if (2 * (wave & 1) < ((wave >> 1) ? ntf1 : ntf0)) {
-                ld.sc_base = reinterpret_cast<const char *>(tok_sc_base);
-                ld.sc_off = tok_sc_off(row);
-                ld.sc_step = 4u;
-                ld.sc_dst = C::kScaleOff + 64 * wave * 4;
-            }
+            ld.sc_dst = lay.scale_off + (lay.scale_tok_rows + 64 * (wave - 4)) * 4;
+        } else if (64 * wave < lay.tok_rows) {
+            // packed token rows 64 wave + lane (the lanes past the last live row repeat it)
+            const int c = min(64 * wave + lane, lay.tok_rows - 1);
+            const int row = c < 32 * ntf0 ? c : kBlockRows + c - 32 * ntf0;
+            ld.sc_base = reinterpret_cast<const char *>(tok_sc_base);
+            ld.sc_off = tok_sc_off(row);
+            ld.sc_step = 4u;
+            ld.sc_dst = lay.scale_off + 64 * wave * 4;
         }
     }
     ld.lps = 2 + (ld.tok_dst[0] >= 0) + (ld.tok_dst[1] >= 0) + (ld.sc_dst >= 0);
@@ -333,11 +283,11 @@ __device__ __forceinline__ int slab_rotation(int n_slabs) {
     return phase % n_slabs & ~1;
 }
 
-// Up kernel tile: two row blocks (SKINNY: one block with at most 32 live rows) x activation columns
-// [128 ht, 128 ht + 128).  LDS weight rows 0..127 are gate rows, 128..255 the matching up rows; wave
-// v of a group owns gate/up rows 32v..32v+31 so gate and up of one activation element sit in the
+// Up kernel tile on the 64-byte ring: the live fragments of one or two row blocks x activation
+// columns [128 ht, 128 ht + 128).  LDS weight rows 0..127 are gate rows, 128..255 the matching up rows;
+// wave v of a group owns gate/up rows 32v..32v+31 so gate and up of one activation element sit in the
 // same lane and register.
-template <int DT, bool SKINNY, int NTF, bool FULL>
+template <int DT, int NTF, bool FULL>
 __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht, int e, RowInfo<2> &ri,
                                              char *lds, uint32_t *act_sc_lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
@@ -349,6 +299,7 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
     const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
     const int my_ntf = grp ? ntf1 : ntf0;
     const bool active = my_ntf > 0;
+    const ring::Layout lay = ring::make_layout<DT>(ntf0, ntf1, ring::ring_bytes<DT>());
 
     ring::Loader ld;
     ld.tok_base = a.x;
@@ -356,8 +307,8 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
     ld.w_base[1] = ld.w_base[0] + (int64_t)H * K * ES;
     const uint32_t row_bytes = (uint32_t)(K * ES);
     const int kb = K >> 5;
-    setup_ring_loader<DT, SKINNY>(
-        ld, tid, row_bytes, ntf0, ntf1,
+    setup_ring_loader<DT>(
+        ld, lay, tid, row_bytes, ntf0, ntf1,
         [&](int row) { return (uint32_t)max(ri.tok[row], 0) * row_bytes; },  // dead rows read token 0
         a.x_scales, [&](int row) { return (uint32_t)max(ri.tok[row], 0) * (uint32_t)kb; },
         a.w1_scales + (int64_t)e * N * kb,
@@ -368,15 +319,15 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
     zero_acc(acc);
     const int n_slabs = (K * ES) / ring::kRB;
     const int start = slab_rotation(n_slabs);
-    const int tok_region = SKINNY ? 0 : grp * ring::kGroupRegion;
-    if (active) ring::main_loop<DT, SKINNY, NTF, true, true, FULL>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
-    else ring::main_loop<DT, SKINNY, NTF, true, false, FULL>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
+    const int tok_region = grp ? lay.group1_off : 0;
+    if (active) ring::main_loop<DT, NTF, true, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
+    else ring::main_loop<DT, NTF, true, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
 
     // the ring is free (main_loop ends with a barrier): reuse it for the activation tiles
     constexpr int kPitch = DT == DT_BF16 ? kActPitchBf16 : kActPitchFp8;
     char *tile = lds + grp * (kBlockRows * kPitch);
     uint32_t *sc_tile = act_sc_lds + grp * kBlockRows;
-    if (active) swiglu_epilogue<DT, false, NTF>(acc, tile, sc_tile, w4, lane);
+    if (active) swiglu_epilogue<DT, NTF>(acc, tile, sc_tile, w4, lane);
     __syncthreads();
     if (active) store_act_tile<DT>(a, tile, sc_tile, (int64_t)(first + grp) * kBlockRows, h0, my_ntf, gt);
 }
@@ -393,7 +344,7 @@ struct SplitLds {
     static constexpr int kActScaleOff = kRowInfoOff + kRowInfoBytes;  // mxfp8 only
     static constexpr int kTotal = DT == DT_BF16 ? kRing : kActScaleOff + kBlockRows * 2 * 4;
     static_assert(sizeof(RowInfo<2>) <= kRowInfoBytes, "row table does not fit its slot");
-    static_assert(DT != DT_BF16 || ring::Cfg<DT_BF16, true>::kRingBytes <= kRowInfoOff, "skinny ring reaches the row table");
+    static_assert(DT != DT_BF16 || ring::ring_bytes<DT_BF16>() <= kRowInfoOff, "64-byte ring reaches the row table");
 };
 
 // First slab of a wide bf16 tile's walk over K: 8 phases, one 128-byte slab apart.
@@ -427,7 +378,7 @@ __device__ __forceinline__ void up_tile_wide_bf16(const MoeArgs &a, int first, i
     else ring128::main_loop<NTF, true, false>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
 
     char *tile = lds + grp * (kBlockRows * kActPitchBf16);
-    if (active) swiglu_epilogue<DT_BF16, false, NTF>(acc, tile, nullptr, w4, lane);
+    if (active) swiglu_epilogue<DT_BF16, NTF>(acc, tile, nullptr, w4, lane);
     __syncthreads();
     if (active) store_act_tile<DT_BF16>(a, tile, nullptr, (int64_t)(first + grp) * kBlockRows, h0, my_ntf, gt);
 }
@@ -438,7 +389,7 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
     __shared__ __attribute__((aligned(1024))) char lds[L::kTotal];
     RowInfo<2> &ri = *reinterpret_cast<RowInfo<2> *>(lds + L::kRowInfoOff);
     int first, nb, ht;
-    if (!resolve_tile<2>(a, first, nb, ht)) return;
+    if (!resolve_tile(a, first, nb, ht)) return;
     if (first * kBlockRows >= a.ntpp[0]) return;
     const int ntf = load_row_info<2>(a, first, nb, ri);
     if (ntf == 0) return;
@@ -446,24 +397,23 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
     if (e < 0 || e >= a.E) return;
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {
-        if (skinny) up_tile_ring<DT, true, 1, false>(a, first, ht, e, ri, lds, nullptr);
+        if (skinny) up_tile_ring<DT, 1, false>(a, first, ht, e, ri, lds, nullptr);
         else if (ntf == 1) up_tile_wide_bf16<1>(a, first, ht, e, ri, lds);
         else if (ntf == 2) up_tile_wide_bf16<2>(a, first, ht, e, ri, lds);
         else up_tile_wide_bf16<4>(a, first, ht, e, ri, lds);
     } else {
         uint32_t *act_sc_lds = reinterpret_cast<uint32_t *>(lds + L::kActScaleOff);
         const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-        if (skinny) up_tile_ring<DT, true, 1, false>(a, first, ht, e, ri, lds, act_sc_lds);
-        else if (ntf == 1) up_tile_ring<DT, false, 1, false>(a, first, ht, e, ri, lds, act_sc_lds);
-        else if (ntf == 2) up_tile_ring<DT, false, 2, false>(a, first, ht, e, ri, lds, act_sc_lds);
-        else if (full) up_tile_ring<DT, false, 4, true>(a, first, ht, e, ri, lds, act_sc_lds);
-        else up_tile_ring<DT, false, 4, false>(a, first, ht, e, ri, lds, act_sc_lds);
+        if (ntf == 1) up_tile_ring<DT, 1, false>(a, first, ht, e, ri, lds, act_sc_lds);
+        else if (ntf == 2) up_tile_ring<DT, 2, false>(a, first, ht, e, ri, lds, act_sc_lds);
+        else if (full) up_tile_ring<DT, 4, true>(a, first, ht, e, ri, lds, act_sc_lds);
+        else up_tile_ring<DT, 4, false>(a, first, ht, e, ri, lds, act_sc_lds);
     }
 }
 
 // Down kernel of the split pipeline: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
 // full reduction over H inside the workgroup (no split-K), then w[row] * y added to accum[token].
-template <int DT, bool SKINNY, int NTF, bool FULL>
+template <int DT, int NTF, bool FULL>
 __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, char *lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -474,6 +424,7 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     const int ntf0 = __builtin_amdgcn_readfirstlane((ri.nvalid[0] + 31) >> 5);
     const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
     const bool active = (grp ? ntf1 : ntf0) > 0;
+    const ring::Layout lay = ring::make_layout<DT>(ntf0, ntf1, ring::ring_bytes<DT>());
 
     ring::Loader ld;
     ld.tok_base = a.act + row0 * H * ES;
@@ -481,8 +432,8 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     ld.w_base[1] = (k0 + 128 < K) ? ld.w_base[0] + (int64_t)128 * H * ES : ld.w_base[0];
     const uint32_t row_bytes = (uint32_t)(H * ES);
     const int hb = H >> 5;
-    setup_ring_loader<DT, SKINNY>(
-        ld, tid, row_bytes, ntf0, ntf1, [&](int row) { return (uint32_t)row * row_bytes; },
+    setup_ring_loader<DT>(
+        ld, lay, tid, row_bytes, ntf0, ntf1, [&](int row) { return (uint32_t)row * row_bytes; },
         a.act_scales + row0 * hb, [&](int row) { return (uint32_t)row * (uint32_t)hb; },
         a.w2_scales + (int64_t)e * K * hb,
         [&](int row) { return (uint32_t)blocked_scale_off(min(k0 + row, K - 1), 0, H >> 7); });
@@ -492,12 +443,12 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     zero_acc(acc);
     const int n_slabs = (H * ES) / ring::kRB;
     const int start = slab_rotation(n_slabs);
-    const int tok_region = SKINNY ? 0 : grp * ring::kGroupRegion;
+    const int tok_region = grp ? lay.group1_off : 0;
     if (active) {
-        ring::main_loop<DT, SKINNY, NTF, false, true, FULL>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
+        ring::main_loop<DT, NTF, false, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
         scatter_add<NTF>(acc, ri.tok + grp * kBlockRows, ri.wt + grp * kBlockRows, a.accum, K, k0 + 64 * w4, lane);
     } else {
-        ring::main_loop<DT, SKINNY, NTF, false, false, FULL>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
+        ring::main_loop<DT, NTF, false, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
     }
 }
 
@@ -542,7 +493,7 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
     __shared__ __attribute__((aligned(1024))) char lds[L::kTotal];
     RowInfo<2> &ri = *reinterpret_cast<RowInfo<2> *>(lds + L::kRowInfoOff);
     int first, nb, kt;
-    if (!resolve_tile<2>(a, first, nb, kt)) return;
+    if (!resolve_tile(a, first, nb, kt)) return;
     if (first * kBlockRows >= a.ntpp[0]) return;
     const int ntf = load_row_info<2>(a, first, nb, ri);
     if (ntf == 0) return;
@@ -550,218 +501,16 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
     if (e < 0 || e >= a.E) return;
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {
-        if (skinny) down_tile_ring<DT, true, 1, false>(a, first, kt, e, ri, lds);
+        if (skinny) down_tile_ring<DT, 1, false>(a, first, kt, e, ri, lds);
         else if (ntf == 1) down_tile_wide_bf16<1>(a, first, kt, e, ri, lds);
         else if (ntf == 2) down_tile_wide_bf16<2>(a, first, kt, e, ri, lds);
         else down_tile_wide_bf16<4>(a, first, kt, e, ri, lds);
     } else {
         const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-        if (skinny) down_tile_ring<DT, true, 1, false>(a, first, kt, e, ri, lds);
-        else if (ntf == 1) down_tile_ring<DT, false, 1, false>(a, first, kt, e, ri, lds);
-        else if (ntf == 2) down_tile_ring<DT, false, 2, false>(a, first, kt, e, ri, lds);
-        else if (full) down_tile_ring<DT, false, 4, true>(a, first, kt, e, ri, lds);
-        else down_tile_ring<DT, false, 4, false>(a, first, kt, e, ri, lds);
-    }
-}
-
-// ==========================================================================================
-// Fused pipeline (split == 0): one row block per 256-thread workgroup, register-staged engine
-// ==========================================================================================
-
-// K loop of one tile: double-buffered LDS stages, prefetch of slab k+1 while slab k computes.
-template <int DT, int NTF, bool TRANSPOSED>
-__device__ __forceinline__ void tile_main_loop(f32x16 (&acc)[2][4], StageLoader<1> &ld, char *lds,
-                                               int n_slabs, const int (&wrow)[2], int lane,
-                                               const uint8_t *tok_sc_base, const uint32_t (&tok_sc)[4],
-                                               const uint8_t *w_sc_base, const uint32_t (&w_sc)[2]) {
-    using G = Geo<1>;
-    uint32_t stok[4] = {0, 0, 0, 0}, sw[2] = {0, 0};
-    uint32_t ntok[4] = {0, 0, 0, 0}, nw[2] = {0, 0};
-    ld.load_tok(0);
-    ld.load_w(0);
-    if constexpr (DT == DT_FP8) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-            if (t < NTF) stok[t] = *reinterpret_cast<const uint32_t *>(tok_sc_base + tok_sc[t]);
-#pragma unroll
-        for (int f = 0; f < 2; ++f) sw[f] = *reinterpret_cast<const uint32_t *>(w_sc_base + w_sc[f]);
-    }
-    ld.store_tok(lds);
-    ld.store_w(lds);
-    __syncthreads();
-    for (int kt = 0; kt < n_slabs; ++kt) {
-        char *cur = lds + (kt & 1) * G::kStageBytes;
-        char *nxt = lds + ((kt + 1) & 1) * G::kStageBytes;
-        const bool more = kt + 1 < n_slabs;
-        if (more) {
-            ld.load_tok((uint32_t)(kt + 1) * kRowBytes);
-            ld.load_w((uint32_t)(kt + 1) * kRowBytes);
-            if constexpr (DT == DT_FP8) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    if (t < NTF) ntok[t] = *reinterpret_cast<const uint32_t *>(tok_sc_base + (tok_sc[t] + (uint32_t)(kt + 1) * 4));
-#pragma unroll
-                for (int f = 0; f < 2; ++f)
-                    nw[f] = *reinterpret_cast<const uint32_t *>(w_sc_base + (w_sc[f] + (uint32_t)(kt + 1) * 512));
-            }
-        }
-        mfma_slab<DT, NTF, TRANSPOSED, true>(acc, cur, cur + G::kTokRegion, wrow, lane, stok, sw);
-        if (more) {
-            ld.store_tok(nxt);
-            ld.store_w(nxt);
-            if constexpr (DT == DT_FP8) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t) stok[t] = ntok[t];
-#pragma unroll
-                for (int f = 0; f < 2; ++f) sw[f] = nw[f];
-            }
-        }
-        __syncthreads();
-    }
-}
-
-// Up phase of the fused kernel: leaves the SwiGLU (and, for mxfp8, requantised) 128 x 128
-// activation tile in LDS in MFMA operand layout.
-template <int DT, int NTF>
-__device__ __forceinline__ void fused_up_phase(const MoeArgs &a, int ht, int e, RowInfo<1> &ri, char *lds,
-                                               char *act_lds, uint32_t *act_sc_lds) {
-    using G = Geo<1>;
-    constexpr int ES = DT == DT_BF16 ? 2 : 1;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int r = lane & 31;
-    const int K = a.K, H = a.H, N = a.N;
-    const int h0 = ht * 128;
-
-    StageLoader<1> ld;
-    const int lrow = tid >> 3, chunk = tid & 7;
-    ld.lds_off = lrow * kRowBytes + ((chunk ^ swz(lrow)) << 4);
-    ld.tok_mask = 0;
-#pragma unroll
-    for (int i = 0; i < G::kTokPasses; ++i) {
-        const int row = lrow + i * G::kPassRows;
-        ld.tok_off[i] = (uint32_t)max(ri.tok[row], 0) * (uint32_t)(K * ES) + chunk * 16;
-        if ((row >> 5) < ((ri.nvalid[0] + 31) >> 5)) ld.tok_mask |= 1 << i;
-    }
-    ld.tok_mask = __builtin_amdgcn_readfirstlane(ld.tok_mask);  // a wave's 8 rows share a fragment
-    ld.tok_base = a.x;
-    ld.w_base[0] = a.w1 + ((int64_t)e * N + h0) * K * ES;
-    ld.w_base[1] = ld.w_base[0] + (int64_t)H * K * ES;
-    ld.w_off = (uint32_t)lrow * (uint32_t)(K * ES) + chunk * 16;
-    ld.w_pitch_pass = (uint32_t)G::kPassRows * (uint32_t)(K * ES);
-
-    const int wrow[2] = {32 * wave, 128 + 32 * wave};
-    uint32_t tok_sc[4] = {0, 0, 0, 0}, w_sc[2] = {0, 0};
-    const uint8_t *w_sc_base = nullptr;
-    if constexpr (DT == DT_FP8) {
-        const int kb = K >> 5;
-#pragma unroll
-        for (int t = 0; t < 4; ++t) tok_sc[t] = (uint32_t)max(ri.tok[32 * t + r], 0) * (uint32_t)kb;
-        w_sc_base = a.w1_scales + (int64_t)e * N * kb;
-        w_sc[0] = (uint32_t)blocked_scale_off(h0 + 32 * wave + r, 0, K >> 7);
-        w_sc[1] = (uint32_t)blocked_scale_off(H + h0 + 32 * wave + r, 0, K >> 7);
-    }
-    f32x16 acc[2][4];
-    zero_acc(acc);
-    tile_main_loop<DT, NTF, true>(acc, ld, lds, (K * ES) / kRowBytes, wrow, lane, a.x_scales, tok_sc, w_sc_base, w_sc);
-    swiglu_epilogue<DT, true, NTF>(acc, act_lds, act_sc_lds, wave, lane);
-    __syncthreads();
-}
-
-// Down phase of the fused kernel: the activation tile (128 rows x 128 columns of H) stays in
-// LDS as the token operand; W2[e][256-row chunk][h-slice] streams through the weight region.
-template <int DT, int NTF>
-__device__ __forceinline__ void fused_down_phase(const MoeArgs &a, int ht, int e, RowInfo<1> &ri,
-                                                 char *lds, const char *act_lds,
-                                                 const uint32_t *act_sc_lds) {
-    using G = Geo<1>;
-    constexpr int ES = DT == DT_BF16 ? 2 : 1;
-    constexpr int NS = DT == DT_BF16 ? 2 : 1;  // 128-byte slabs across the 128-column h-slice
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int r = lane & 31;
-    const int K = a.K, H = a.H;
-    const int n_chunks = (K + kWRows - 1) / kWRows;
-    const int n_steps = n_chunks * NS;
-
-    StageLoader<1> ld;
-    const int lrow = tid >> 3, chunk = tid & 7;
-    ld.lds_off = lrow * kRowBytes + ((chunk ^ swz(lrow)) << 4);
-    ld.tok_mask = 0;
-    ld.w_pitch_pass = (uint32_t)G::kPassRows * (uint32_t)(H * ES);
-    ld.w_off = (uint32_t)lrow * (uint32_t)(H * ES) + chunk * 16;
-    const char *w2e = a.w2 + (int64_t)e * K * H * ES + (int64_t)ht * 128 * ES;
-    auto set_chunk = [&](int kc) {
-        const int k0 = kc * kWRows;
-        ld.w_base[0] = w2e + (int64_t)k0 * H * ES;
-        ld.w_base[1] = (k0 + 128 < K) ? ld.w_base[0] + (int64_t)128 * H * ES : ld.w_base[0];
-    };
-    const int wrow[2] = {64 * wave, 64 * wave + 32};
-    uint32_t stok[4] = {0, 0, 0, 0}, sw[2] = {0, 0};
-    const uint8_t *w2s = nullptr;
-    if constexpr (DT == DT_FP8) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-            if (t < NTF) stok[t] = act_sc_lds[32 * t + r];
-        w2s = a.w2_scales + (int64_t)e * K * (H >> 5);
-    }
-    auto load_wscales = [&](int kc) {
-        if constexpr (DT == DT_FP8) {
-#pragma unroll
-            for (int f = 0; f < 2; ++f) {
-                int row = kc * kWRows + 64 * wave + 32 * f + r;
-                if (row >= K) row = K - 1;
-                sw[f] = *reinterpret_cast<const uint32_t *>(w2s + blocked_scale_off(row, ht, H >> 7));
-            }
-        }
-    };
-
-    f32x16 acc[2][4];
-    set_chunk(0);
-    ld.load_w(0);
-    ld.store_w(lds);
-    __syncthreads();
-    for (int s = 0; s < n_steps; ++s) {
-        const int kc = s / NS, sl = s - kc * NS;
-        char *cur = lds + (s & 1) * G::kStageBytes;
-        char *nxt = lds + ((s + 1) & 1) * G::kStageBytes;
-        const bool more = s + 1 < n_steps;
-        if (more) {
-            const int nkc = (s + 1) / NS, nsl = (s + 1) - nkc * NS;
-            if (nsl == 0) set_chunk(nkc);
-            ld.load_w((uint32_t)nsl * kRowBytes);
-        }
-        if (sl == 0) {
-            zero_acc(acc);
-            load_wscales(kc);
-        }
-        mfma_slab<DT, NTF, false, true>(acc, act_lds + sl * kGroupRegion, cur + G::kTokRegion, wrow, lane, stok, sw);
-        if (sl == NS - 1) scatter_add<NTF>(acc, ri.tok, ri.wt, a.accum, K, kc * kWRows + 64 * wave, lane);
-        if (more) ld.store_w(nxt);
-        __syncthreads();
-    }
-}
-
-template <int DT>
-__global__ __launch_bounds__(256) void moe_fused_kernel(MoeArgs a) {
-    __shared__ __attribute__((aligned(1024))) char lds[kNumStages * Geo<1>::kStageBytes];
-    __shared__ __attribute__((aligned(1024))) char act_lds[(DT == DT_BF16 ? 2 : 1) * kGroupRegion];
-    __shared__ uint32_t act_sc_lds[kBlockRows];
-    __shared__ RowInfo<1> ri;
-    int first, nb, ht;
-    if (!resolve_tile<1>(a, first, nb, ht)) return;
-    if (first * kBlockRows >= a.ntpp[0]) return;
-    const int ntf = load_row_info<1>(a, first, nb, ri);
-    if (ntf == 0) return;
-    const int e = a.expert_ids[first];
-    if (e < 0 || e >= a.E) return;
-    if (ntf == 1) {
-        fused_up_phase<DT, 1>(a, ht, e, ri, lds, act_lds, act_sc_lds);
-        fused_down_phase<DT, 1>(a, ht, e, ri, lds, act_lds, act_sc_lds);
-    } else if (ntf == 2) {
-        fused_up_phase<DT, 2>(a, ht, e, ri, lds, act_lds, act_sc_lds);
-        fused_down_phase<DT, 2>(a, ht, e, ri, lds, act_lds, act_sc_lds);
-    } else {
-        fused_up_phase<DT, 4>(a, ht, e, ri, lds, act_lds, act_sc_lds);
-        fused_down_phase<DT, 4>(a, ht, e, ri, lds, act_lds, act_sc_lds);
+        if (ntf == 1) down_tile_ring<DT, 1, false>(a, first, kt, e, ri, lds);
+        else if (ntf == 2) down_tile_ring<DT, 2, false>(a, first, kt, e, ri, lds);
+        else if (full) down_tile_ring<DT, 4, true>(a, first, kt, e, ri, lds);
+        else down_tile_ring<DT, 4, false>(a, first, kt, e, ri, lds);
     }
 }
 
@@ -873,7 +622,7 @@ struct WorkspaceLayout {
     size_t n_tiles_off, tiles_off, work_up_off, work_down_off, accum_off, act_off, act_scales_off, total;
 };
 
-static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_num, int split) {
+static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_num) {
     WorkspaceLayout l{};
     const size_t H = (size_t)N / 2;
     const size_t rows = align_up((size_t)sorted_num, kBlockRows);
@@ -884,18 +633,15 @@ static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_
     l.tiles_off = off;
     off = align_up(off + blocks * sizeof(int2), 256);
     l.work_up_off = off;
-    if (split) off = align_up(off + blocks * (H / 128) * sizeof(int2), 256);
+    off = align_up(off + blocks * (H / 128) * sizeof(int2), 256);
     l.work_down_off = off;
-    if (split) off = align_up(off + blocks * (((size_t)K + kWRows - 1) / kWRows) * sizeof(int2), 256);
+    off = align_up(off + blocks * (((size_t)K + kWRows - 1) / kWRows) * sizeof(int2), 256);
     l.accum_off = off;
     off = align_up(off + (size_t)M * K * sizeof(float), 256);
     l.act_off = off;
+    off = align_up(off + rows * H * (dt == DT_BF16 ? 2 : 1), 256);
     l.act_scales_off = off;
-    if (split) {
-        off = align_up(off + rows * H * (dt == DT_BF16 ? 2 : 1), 256);
-        l.act_scales_off = off;
-        if (dt == DT_FP8) off = align_up(off + rows * (H / 32), 256);
-    }
+    if (dt == DT_FP8) off = align_up(off + rows * (H / 32), 256);
     l.total = off;
     return l;
 }
@@ -928,23 +674,18 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
         const int do_zero = (mask & PMOE_PHASE_ZERO) ? 1 : 0;
         const int blocks = do_zero ? (int)std::min<int64_t>((n4 + 255) / 256, 2048) : 1;
         hipLaunchKernelGGL(moe_prologue_kernel, dim3(blocks), dim3(256), 0, s, a.expert_ids, a.ntpp, a.n_blocks,
-                           split ? sb.tiles : nullptr, sb.n_tiles, sb.work_up, a.n_wtiles,
+                           sb.tiles, sb.n_tiles, sb.work_up, a.n_wtiles,
                            sb.work_down, n_wt_down, reinterpret_cast<float4 *>(a.accum), n4, do_zero);
     }
     if (a.n_blocks > 0) {
-        const int grid = grid_for(a.n_blocks * a.n_wtiles);
-        if (split) {
-            a.work = sb.work_up;
-            if (mask & PMOE_PHASE_UP)
-                hipLaunchKernelGGL((moe_up_kernel<DT>), dim3(grid), dim3(512), 0, s, a);
-            MoeArgs d = a;
-            d.n_wtiles = n_wt_down;
-            d.work = sb.work_down;
-            if (mask & PMOE_PHASE_DOWN)
-                hipLaunchKernelGGL((moe_down_kernel<DT>), dim3(grid_for(d.n_blocks * d.n_wtiles)), dim3(512), 0, s, d);
-        } else if (mask & PMOE_PHASE_UP) {
-            hipLaunchKernelGGL((moe_fused_kernel<DT>), dim3(grid), dim3(256), 0, s, a);
-        }
+        a.work = sb.work_up;
+        if (mask & PMOE_PHASE_UP)
+            hipLaunchKernelGGL((moe_up_kernel<DT>), dim3(grid_for(a.n_blocks * a.n_wtiles)), dim3(512), 0, s, a);
+        MoeArgs d = a;
+        d.n_wtiles = n_wt_down;
+        d.work = sb.work_down;
+        if (mask & PMOE_PHASE_DOWN)
+            hipLaunchKernelGGL((moe_down_kernel<DT>), dim3(grid_for(d.n_blocks * d.n_wtiles)), dim3(512), 0, s, d);
     }
     if (mask & PMOE_PHASE_FINALIZE) {
         const int64_t n8 = n_out / 8;
@@ -978,14 +719,14 @@ extern "C" size_t pmoe_fused_moe_bf16_workspace_bytes(int M, int K, int N, int n
                                                       int sorted_num, int split) {
     (void)num_experts;
     if (M <= 0 || K <= 0 || N <= 0 || sorted_num < 0) return 0;
-    return workspace_layout(DT_BF16, M, K, N, sorted_num, split).total;
+    return workspace_layout(DT_BF16, M, K, N, sorted_num).total;
 }
 
 extern "C" size_t pmoe_fused_moe_mxfp8_workspace_bytes(int M, int K, int N, int num_experts,
                                                        int sorted_num, int split) {
     (void)num_experts;
     if (M <= 0 || K <= 0 || N <= 0 || sorted_num < 0) return 0;
-    return workspace_layout(DT_FP8, M, K, N, sorted_num, split).total;
+    return workspace_layout(DT_FP8, M, K, N, sorted_num).total;
 }
 
 static int check_tuning(const char *op, int block_m, int block_n, int warp_n, int stages,
@@ -1012,7 +753,7 @@ extern "C" int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2,
     PMOE_REQUIRE(top_k > 0 && num_experts > 0 && sorted_num >= 0, "fused_moe_bf16: bad top_k / num_experts / sorted_num");
     PMOE_REQUIRE(x && w && w2 && out && sorted_token_ids && expert_idxs && num_tokens_post_padded && topk_weights,
                  "fused_moe_bf16: null pointer");
-    const WorkspaceLayout l = workspace_layout(DT_BF16, M, K, N, sorted_num, split);
+    const WorkspaceLayout l = workspace_layout(DT_BF16, M, K, N, sorted_num);
     PMOE_REQUIRE(workspace && workspace_bytes >= l.total, "fused_moe_bf16: workspace of %zu bytes needed, got %zu", l.total, workspace_bytes);
     PMOE_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, "fused_moe_bf16: workspace must be 256-byte aligned");
     MoeArgs a{};
@@ -1047,7 +788,7 @@ extern "C" int pmoe_fused_moe_mxfp8(const void *x, const void *x_scales, const v
     PMOE_REQUIRE(x && x_scales && w && w_scales && w2 && w2_scales && out && sorted_token_ids && expert_idxs &&
                      num_tokens_post_padded && topk_weights,
                  "fused_moe_mxfp8: null pointer");
-    const WorkspaceLayout l = workspace_layout(DT_FP8, M, K, N, sorted_num, split);
+    const WorkspaceLayout l = workspace_layout(DT_FP8, M, K, N, sorted_num);
     PMOE_REQUIRE(workspace && workspace_bytes >= l.total, "fused_moe_mxfp8: workspace of %zu bytes needed, got %zu", l.total, workspace_bytes);
     PMOE_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, "fused_moe_mxfp8: workspace must be 256-byte aligned");
     MoeArgs a{};

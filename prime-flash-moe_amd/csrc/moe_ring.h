@@ -5,14 +5,17 @@
 // (global_load_lds_*: no staging registers, no ds_write) into a ring of stages; all but one stage
 // are in flight while one is consumed.  One barrier per slab.
 //
-// Two layouts of the ring share the code:
-//   WIDE   256 token rows (two sorted blocks, one per group of 4 waves), 4 stages of 32 KB (+2 KB
-//          of scales for mxfp8): the compute-bound shapes; 96 KB in flight per CU.
-//   SKINNY 32 token rows (a single block with at most 32 live rows: decode), 8 stages of 18 KB
-//          (+1.25 KB): the tile is almost only weights, and seven stages = 126 KB of weight rows in
-//          flight per CU are what it takes to keep HBM busy (latency x bandwidth per CU ~ 60 KB).
+// The ring is sized per tile.  A stage holds only the 32-row token fragments that have live rows
+// (group 0's first, then group 1's), the 256 weight rows and, for mxfp8, the scale dwords of both;
+// as many stages as fit the LDS budget are used, at most 8:
+//   two full blocks (256 token rows)       4 stages of 32 KB (+2 KB scales), 96 KB in flight per CU;
+//   one full block (128 token rows)        6 stages of 24 KB (+1.5 KB), 80 KB of weight rows in flight;
+//   a decode tile (32 live rows)           8 stages of 18 KB (+1.25 KB), 112 KB of weight rows in flight.
+// The fewer token rows a tile has, the closer it is to a pure stream of weights from HBM, and what
+// keeps HBM busy then is weight bytes in flight per CU (latency x bandwidth per CU ~ 60 KB).
 //
-// Stage layout: [token rows][64 B] [256 weight rows][64 B] [scale dwords of all rows (mxfp8)].
+// Stage layout: [live token rows][64 B] [256 weight rows][64 B] [scale dwords: token rows rounded up
+// to a multiple of 64, then weight rows (mxfp8)].
 // A row is 4 chunks of 16 B; chunk c of row r sits in slot c ^ ((r >> 2) & 3): the 16-byte MFMA
 // operand reads of 16 consecutive rows then cover all 64 LDS banks exactly once.  The copy engine
 // writes lane l of a wave instruction to bytes [16 l, 16 l + 16) behind a wave-uniform base, so the
@@ -35,22 +38,45 @@ namespace ring {
 
 constexpr int kRB = 64;  // row bytes of a slab
 
-template <int DT, bool SKINNY>
-struct Cfg {
-    static constexpr int kStages = SKINNY ? 8 : 4;
-    static constexpr int kTokRows = SKINNY ? 32 : 256;
-    static constexpr int kTokRegion = kTokRows * kRB;
-    static constexpr int kWRegion = kWRows * kRB;  // 16 KB
-    static constexpr int kScaleOff = kTokRegion + kWRegion;
-    static constexpr int kScaleTokRows = SKINNY ? 64 : 256;  // token scale dwords (a whole wave instruction)
-    static constexpr int kStageBytes = kScaleOff + (DT == DT_FP8 ? (kScaleTokRows + kWRows) * 4 : 0);
-    static constexpr int kRingBytes = kStages * kStageBytes;
+constexpr int kMaxStages = 8;
+
+// Geometry of a tile's ring; every member is wave-uniform.
+struct Layout {
+    int tok_rows;        // live token rows of both groups: 32 (ntf0 + ntf1)
+    int group1_off;      // byte offset of group 1's token rows inside a stage
+    int w_off;           // byte offset of the weight rows
+    int scale_off;       // byte offset of the scale dwords (mxfp8)
+    int scale_tok_rows;  // token scale dwords reserved: tok_rows rounded up to 64
+    int stage_bytes;
+    int stages;
 };
 template <int DT>
-constexpr int ring_bytes() {
-    return Cfg<DT, true>::kRingBytes > Cfg<DT, false>::kRingBytes ? Cfg<DT, true>::kRingBytes : Cfg<DT, false>::kRingBytes;
+__device__ __forceinline__ Layout make_layout(int ntf0, int ntf1, int budget) {
+    Layout l;
+    l.tok_rows = 32 * (ntf0 + ntf1);
+    l.group1_off = 32 * ntf0 * kRB;
+    l.w_off = l.tok_rows * kRB;
+    l.scale_off = l.w_off + kWRows * kRB;
+    l.scale_tok_rows = (l.tok_rows + 63) & ~63;
+    const int bytes = l.scale_off + (DT == DT_FP8 ? (l.scale_tok_rows + kWRows) * 4 : 0);
+    l.stage_bytes = (bytes + 255) & ~255;
+    l.stages = min(kMaxStages, budget / l.stage_bytes);
+    return l;
 }
-constexpr int kGroupRegion = kBlockRows * kRB;  // one group's 128 token rows in the wide layout
+// Compile-time geometry of the tile with two full blocks (4 stages).
+template <int DT>
+struct FullCfg {
+    static constexpr int kStages = 4;
+    static constexpr int kTokRows = 256;
+    static constexpr int kWOff = kTokRows * kRB;
+    static constexpr int kScaleOff = kWOff + kWRows * kRB;
+    static constexpr int kStageBytes = kScaleOff + (DT == DT_FP8 ? (kTokRows + kWRows) * 4 : 0);
+};
+// LDS the ring may use, a multiple of 1 KB (the split kernels put their row table behind it).
+template <int DT>
+constexpr int ring_bytes() {
+    return DT == DT_FP8 ? 156 * 1024 : 144 * 1024;
+}
 
 __device__ __forceinline__ int swz64(int row) { return (row >> 2) & 3; }
 
@@ -74,16 +100,16 @@ template <int N>
 __device__ __forceinline__ void wait_and_barrier() {
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
 }
-// Waits until at most `n` (wave-uniform, <= 28) of this wave's copies are in flight and its LDS
+// Waits until at most `n` (wave-uniform, <= 30) of this wave's copies are in flight and its LDS
 // reads have returned, then joins the workgroup barrier.  The wait count is an immediate of the
-// instruction, hence the switch.
+// instruction, hence the switch (at most 5 copies per stage x 6 stages behind the current one).
 __device__ __forceinline__ void wait_and_barrier_dyn(int n) {
     switch (n) {
 #define PMOE_WB(k) case k: wait_and_barrier<k>(); break;
         PMOE_WB(1) PMOE_WB(2) PMOE_WB(3) PMOE_WB(4) PMOE_WB(5) PMOE_WB(6) PMOE_WB(7) PMOE_WB(8) PMOE_WB(9)
         PMOE_WB(10) PMOE_WB(11) PMOE_WB(12) PMOE_WB(13) PMOE_WB(14) PMOE_WB(15) PMOE_WB(16) PMOE_WB(17)
         PMOE_WB(18) PMOE_WB(19) PMOE_WB(20) PMOE_WB(21) PMOE_WB(22) PMOE_WB(23) PMOE_WB(24) PMOE_WB(25)
-        PMOE_WB(26) PMOE_WB(27) PMOE_WB(28)
+        PMOE_WB(26) PMOE_WB(27) PMOE_WB(28) PMOE_WB(29) PMOE_WB(30)
 #undef PMOE_WB
         default: wait_and_barrier<0>(); break;
     }
@@ -195,29 +221,30 @@ __device__ __forceinline__ void mma_fp8_slab(f32x16 (&acc)[2][4], const char *to
 }
 
 // K loop.  COMPUTE = false is the loop of the waves without matrix work (a group without live
-// rows; waves 4-7 of a skinny tile): they only issue their share of the copies and join the
-// barriers.  `tok_region` = byte offset of this wave's token rows inside a stage.
+// rows): they only issue their share of the copies and join the barriers.  `tok_region` = byte
+// offset of this wave's group inside a stage's token rows.
 //
 // The slabs are visited in rotated order, starting at slab `start` (even): workgroups that run
 // side by side and share rows then ask for different cache lines at any one time instead of
 // queueing on the same ones.  The sum over K does not depend on the order.
 //
-// FULL: every wave of the workgroup issues the maximum number of copies per stage (a wide tile whose
-// two blocks are completely live), so the wait counts are compile-time constants; otherwise they
-// are computed per wave and dispatched through a switch.
-template <int DT, bool SKINNY, int NTF, bool TRANSPOSED, bool COMPUTE, bool FULL>
-__device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader &ld, char *lds, int n_slabs,
-                                          const int (&wrow)[2], int lane, int tok_region, int start) {
-    using C = Cfg<DT, SKINNY>;
-    constexpr int SB = C::kStageBytes;
-    constexpr int NS = C::kStages;
+// FULL: the tile has two completely live blocks, so geometry and wait counts are compile-time
+// constants (`lay` must be that geometry); otherwise both are wave-uniform run-time values and the
+// wait count goes through a switch.
+template <int DT, int NTF, bool TRANSPOSED, bool COMPUTE, bool FULL>
+__device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader &ld, const Layout &lay, char *lds,
+                                          int n_slabs, const int (&wrow)[2], int lane, int tok_region, int start) {
+    using F = FullCfg<DT>;
+    const int SB = FULL ? F::kStageBytes : lay.stage_bytes;
+    const int NS = FULL ? F::kStages : lay.stages;
+    const int w_off = FULL ? F::kWOff : lay.w_off;
+    const int scale_off = FULL ? F::kScaleOff : lay.scale_off;
+    const int scale_tok_rows = FULL ? F::kTokRows : lay.scale_tok_rows;
     constexpr int LPS_FULL = DT == DT_FP8 ? 5 : 4;
-    static_assert(!FULL || (!SKINNY && NS == 4), "constant wait counts are written for the 4-stage ring");
     auto rot = [&](int s) {
         s += start;
         return s >= n_slabs ? s - n_slabs : s;
     };
-#pragma unroll
     for (int s = 0; s < NS - 1; ++s)
         if (s < n_slabs) ld.issue(lds + s * SB, rot(s));
     FragsBf16 fx, fy;  // fy carries the held-back sub-step across the barrier
@@ -232,6 +259,8 @@ __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader &ld,
             for (int i = 0; i < 8; ++i) fy.b[t][i] = (__bf16)0.0f;
     }
     const int lps = ld.lps;
+    int cur_off = 0;               // stage of slab kt
+    int fill_off = (NS - 1) * SB;  // stage slab kt + NS - 1 goes to (the one slab kt - 1 used)
     for (int kt = 0; kt < n_slabs; ++kt) {
         // slab kt has landed once at most the copies of the later slabs (up to NS - 2) are pending
         if constexpr (FULL) {
@@ -242,11 +271,11 @@ __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader &ld,
             wait_and_barrier_dyn(lps * min(NS - 2, n_slabs - 1 - kt));
         }
         // the stage consumed in the previous iteration is free: everybody is past the barrier
-        if (kt + NS - 1 < n_slabs) ld.issue(lds + ((kt + NS - 1) & (NS - 1)) * SB, rot(kt + NS - 1));
+        if (kt + NS - 1 < n_slabs) ld.issue(lds + fill_off, rot(kt + NS - 1));
         if constexpr (COMPUTE) {
-            const char *cur = lds + (kt & (NS - 1)) * SB;
+            const char *cur = lds + cur_off;
             const char *tok = cur + tok_region;
-            const char *wgt = cur + C::kTokRegion;
+            const char *wgt = cur + w_off;
             if constexpr (DT == DT_BF16) {
                 // software pipeline across the barrier: the second K sub-step of a slab is held back
                 // and issued behind the first fragment reads of the next slab
@@ -254,26 +283,16 @@ __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader &ld,
                 mma_bf16<NTF, TRANSPOSED>(acc, fy);
                 fetch_bf16<NTF>(fy, tok, wgt, wrow, lane, 1);
                 mma_bf16<NTF, TRANSPOSED>(acc, fx);
-                if constexpr (NTF == 4) {
-                    // issue order: the 8 MFMAs of one fragment buffer alternate with the 6 LDS reads
-                    // that refill the other
-#pragma unroll
-                    for (int p = 0; p < 2; ++p) {
-#pragma unroll
-                        for (int i = 0; i < 6; ++i) {
-                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                        }
-                        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-                    }
-                }
             } else {
-                const uint32_t *sc = reinterpret_cast<const uint32_t *>(cur + C::kScaleOff);
+                const uint32_t *sc = reinterpret_cast<const uint32_t *>(cur + scale_off);
                 // start is even: the parity of kt is the parity of the slab inside its 128-wide K tile
-                mma_fp8_slab<NTF, TRANSPOSED>(acc, tok, wgt, sc + tok_region / kRB, sc + C::kScaleTokRows, wrow, lane,
+                mma_fp8_slab<NTF, TRANSPOSED>(acc, tok, wgt, sc + tok_region / kRB, sc + scale_tok_rows, wrow, lane,
                                               8 * (2 * (kt & 1) + (lane >> 5)));
             }
         }
+        fill_off = cur_off;
+        cur_off += SB;
+        if (cur_off >= NS * SB) cur_off = 0;
     }
     if constexpr (DT == DT_BF16 && COMPUTE) mma_bf16<NTF, TRANSPOSED>(acc, fy);
     __syncthreads();  // all reads of the last stages are done: the ring may be reused as scratch

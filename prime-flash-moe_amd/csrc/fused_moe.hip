@@ -44,6 +44,15 @@ struct MoeArgs {
     int n_wtiles;  // weight tiles along the free dimension: H/128 (up) or ceil(K/256) (down)
 };
 
+#ifndef PMOE_SKINNY_RB
+#define PMOE_SKINNY_RB 128
+#endif
+#ifndef PMOE_PART_RB
+#define PMOE_PART_RB 128
+#endif
+constexpr int kSkinnyRB = PMOE_SKINNY_RB;  // slab width of tiles with one live fragment
+constexpr int kPartRB = PMOE_PART_RB;      // of mxfp8 tiles with more, short of two full blocks
+
 constexpr int kActPitchBf16 = 272;  // 128 bf16 + 16 B pad: 16-byte aligned rows, 2-way conflicts at most
 constexpr int kActPitchFp8 = 144;   // 128 e4m3 + 16 B pad
 
@@ -222,32 +231,38 @@ __device__ __forceinline__ void store_act_tile(const MoeArgs &a, const char *til
 // Two-group kernels on the ring engines
 // ==========================================================================================
 
-// Common set-up of the ring loader.  Token rows: `tok_row_off(row)` gives the byte offset of tile
-// row `row` (0..255: block 0, then block 1) in `tok_base`; weight rows: the tile's two 128-row halves
-// start at w_base[0/1] with `w_pitch` bytes per row.  Scales (mxfp8): `tok_sc_off(row)` /
+// Common set-up of the stage-ring loader.  Token rows: `tok_row_off(row)` gives the byte offset of
+// tile row `row` (0..255: block 0, then block 1) in `tok_base`; weight rows: the tile's two 128-row
+// halves start at w_base[0/1] with `w_pitch` bytes per row.  Scales (mxfp8): `tok_sc_off(row)` /
 // `w_sc_off(row)` are the byte offsets of the row's first 4-scale dword.  Only the live 32-row
 // fragments of the two blocks (ntf0, ntf1 of them) are copied; they are packed one after the other in
 // the stage (see ring::Layout).
-template <int DT, typename TokOff, typename TokScOff, typename WScOff>
-__device__ __forceinline__ void setup_ring_loader(ring::Loader &ld, const ring::Layout &lay, int tid, uint32_t w_pitch,
-                                                  int ntf0, int ntf1, TokOff tok_row_off, const uint8_t *tok_sc_base,
-                                                  TokScOff tok_sc_off, const uint8_t *w_sc_base, WScOff w_sc_off) {
+template <int DT, int RB, typename TokOff, typename TokScOff, typename WScOff>
+__device__ __forceinline__ void setup_ring_loader(ring::Loader<RB> &ld, const ring::Layout &lay, int tid,
+                                                  uint32_t w_pitch, int ntf0, int ntf1, TokOff tok_row_off,
+                                                  const uint8_t *tok_sc_base, TokScOff tok_sc_off,
+                                                  const uint8_t *w_sc_base, WScOff w_sc_off) {
+    using L = ring::Loader<RB>;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-    const int prow = tid >> 2;                         // row inside a 128-row pass
-    const int gchunk = (tid & 3) ^ ring::swz64(prow);  // global chunk landing in this lane's LDS slot
-    ld.w_off = (uint32_t)prow * w_pitch + gchunk * 16;
-    ld.w_dst[0] = lay.w_off + wave * 16 * ring::kRB;
-    ld.w_dst[1] = ld.w_dst[0] + 128 * ring::kRB;
-    ld.tok_dst[0] = ld.tok_dst[1] = -1;
-    ld.tok_off[0] = ld.tok_off[1] = 0;
-    const int frag = wave >> 1;  // the wave's 16 rows of a block lie in this fragment
-    if (frag < ntf0) {
-        ld.tok_dst[0] = wave * 16 * ring::kRB;
-        ld.tok_off[0] = tok_row_off(prow) + gchunk * 16;
-    }
-    if (frag < ntf1) {
-        ld.tok_dst[1] = lay.group1_off + wave * 16 * ring::kRB;
-        ld.tok_off[1] = tok_row_off(kBlockRows + prow) + gchunk * 16;
+#pragma unroll
+    for (int q = 0; q < L::N; ++q) {
+        const int row = L::row_of(wave, lane, q);          // row inside a 128-row block / half
+        const int row0 = L::row_of(wave, 0, q);            // first row of the instruction
+        const uint32_t gchunk = (uint32_t)((lane % (RB / 16)) ^ ring::swz<RB>(row)) * 16u;  // global chunk of this lane's slot
+        ld.w_off[q] = (uint32_t)row * w_pitch + gchunk;
+        ld.w_dst[0][q] = lay.w_off + row0 * RB;
+        ld.w_dst[1][q] = ld.w_dst[0][q] + 128 * RB;
+        const int frag = row0 >> 5;  // the instruction's rows lie in this 32-row fragment
+        ld.tok_dst[0][q] = ld.tok_dst[1][q] = -1;
+        ld.tok_off[0][q] = ld.tok_off[1][q] = 0;
+        if (frag < ntf0) {
+            ld.tok_dst[0][q] = row0 * RB;
+            ld.tok_off[0][q] = tok_row_off(row) + gchunk;
+        }
+        if (frag < ntf1) {
+            ld.tok_dst[1][q] = lay.group1_off + row0 * RB;
+            ld.tok_off[1][q] = tok_row_off(kBlockRows + row) + gchunk;
+        }
     }
     ld.sc_base = nullptr;
     ld.sc_off = 0;
@@ -270,7 +285,10 @@ __device__ __forceinline__ void setup_ring_loader(ring::Loader &ld, const ring::
             ld.sc_dst = lay.scale_off + 64 * wave * 4;
         }
     }
-    ld.lps = 2 + (ld.tok_dst[0] >= 0) + (ld.tok_dst[1] >= 0) + (ld.sc_dst >= 0);
+    int lps = 2 * L::N + (ld.sc_dst >= 0);
+#pragma unroll
+    for (int q = 0; q < L::N; ++q) lps += (ld.tok_dst[0][q] >= 0) + (ld.tok_dst[1][q] >= 0);
+    ld.lps = lps;
     ld.make_uniform();
 }
 
@@ -278,16 +296,18 @@ __device__ __forceinline__ void setup_ring_loader(ring::Loader &ld, const ring::
 // blockIdx / 8) start 128 bytes apart, 8 distinct phases over a 1 KB period.  The spread keeps the
 // workgroups that share a weight tile off the same HBM channel at the same instant, and stays short
 // enough that they still meet in L2 (a 16-phase, 4 KB spread read 30 % more from HBM for the same time).
+// Even for 64-byte slabs: two of them share a scale dword.
+template <int RB>
 __device__ __forceinline__ int slab_rotation(int n_slabs) {
-    const int phase = (int)((blockIdx.x >> 3) & 7) * (128 / ring::kRB);
-    return phase % n_slabs & ~1;
+    const int phase = (int)((blockIdx.x >> 3) & 7) * (128 / RB);
+    return RB == 64 ? phase % n_slabs & ~1 : phase % n_slabs;
 }
 
-// Up kernel tile on the 64-byte ring: the live fragments of one or two row blocks x activation
+// Up kernel tile on the stage ring: the live fragments of one or two row blocks x activation
 // columns [128 ht, 128 ht + 128).  LDS weight rows 0..127 are gate rows, 128..255 the matching up rows;
 // wave v of a group owns gate/up rows 32v..32v+31 so gate and up of one activation element sit in the
 // same lane and register.
-template <int DT, int NTF, bool FULL>
+template <int DT, int RB, int NTF, bool FULL>
 __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht, int e, RowInfo<2> &ri,
                                              char *lds, uint32_t *act_sc_lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
@@ -299,15 +319,15 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
     const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
     const int my_ntf = grp ? ntf1 : ntf0;
     const bool active = my_ntf > 0;
-    const ring::Layout lay = ring::make_layout<DT>(ntf0, ntf1, ring::ring_bytes<DT>());
+    const ring::Layout lay = ring::make_layout<DT, RB>(ntf0, ntf1, ring::ring_bytes<DT>());
 
-    ring::Loader ld;
+    ring::Loader<RB> ld;
     ld.tok_base = a.x;
     ld.w_base[0] = a.w1 + ((int64_t)e * N + h0) * K * ES;
     ld.w_base[1] = ld.w_base[0] + (int64_t)H * K * ES;
     const uint32_t row_bytes = (uint32_t)(K * ES);
     const int kb = K >> 5;
-    setup_ring_loader<DT>(
+    setup_ring_loader<DT, RB>(
         ld, lay, tid, row_bytes, ntf0, ntf1,
         [&](int row) { return (uint32_t)max(ri.tok[row], 0) * row_bytes; },  // dead rows read token 0
         a.x_scales, [&](int row) { return (uint32_t)max(ri.tok[row], 0) * (uint32_t)kb; },
@@ -317,11 +337,11 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
     const int wrow[2] = {32 * w4, 128 + 32 * w4};
     f32x16 acc[2][4];
     zero_acc(acc);
-    const int n_slabs = (K * ES) / ring::kRB;
-    const int start = slab_rotation(n_slabs);
+    const int n_slabs = (K * ES) / RB;
+    const int start = slab_rotation<RB>(n_slabs);
     const int tok_region = grp ? lay.group1_off : 0;
-    if (active) ring::main_loop<DT, NTF, true, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
-    else ring::main_loop<DT, NTF, true, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
+    if (active) ring::main_loop<DT, RB, NTF, true, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
+    else ring::main_loop<DT, RB, NTF, true, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
 
     // the ring is free (main_loop ends with a barrier): reuse it for the activation tiles
     constexpr int kPitch = DT == DT_BF16 ? kActPitchBf16 : kActPitchFp8;
@@ -397,23 +417,23 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
     if (e < 0 || e >= a.E) return;
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {
-        if (skinny) up_tile_ring<DT, 1, false>(a, first, ht, e, ri, lds, nullptr);
+        if (skinny) up_tile_ring<DT, kSkinnyRB, 1, false>(a, first, ht, e, ri, lds, nullptr);
         else if (ntf == 1) up_tile_wide_bf16<1>(a, first, ht, e, ri, lds);
         else if (ntf == 2) up_tile_wide_bf16<2>(a, first, ht, e, ri, lds);
         else up_tile_wide_bf16<4>(a, first, ht, e, ri, lds);
     } else {
         uint32_t *act_sc_lds = reinterpret_cast<uint32_t *>(lds + L::kActScaleOff);
         const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-        if (ntf == 1) up_tile_ring<DT, 1, false>(a, first, ht, e, ri, lds, act_sc_lds);
-        else if (ntf == 2) up_tile_ring<DT, 2, false>(a, first, ht, e, ri, lds, act_sc_lds);
-        else if (full) up_tile_ring<DT, 4, true>(a, first, ht, e, ri, lds, act_sc_lds);
-        else up_tile_ring<DT, 4, false>(a, first, ht, e, ri, lds, act_sc_lds);
+        if (ntf == 1) up_tile_ring<DT, kSkinnyRB, 1, false>(a, first, ht, e, ri, lds, act_sc_lds);
+        else if (ntf == 2) up_tile_ring<DT, kPartRB, 2, false>(a, first, ht, e, ri, lds, act_sc_lds);
+        else if (full) up_tile_ring<DT, 64, 4, true>(a, first, ht, e, ri, lds, act_sc_lds);
+        else up_tile_ring<DT, kPartRB, 4, false>(a, first, ht, e, ri, lds, act_sc_lds);
     }
 }
 
 // Down kernel of the split pipeline: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
 // full reduction over H inside the workgroup (no split-K), then w[row] * y added to accum[token].
-template <int DT, int NTF, bool FULL>
+template <int DT, int RB, int NTF, bool FULL>
 __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, char *lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -424,15 +444,15 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     const int ntf0 = __builtin_amdgcn_readfirstlane((ri.nvalid[0] + 31) >> 5);
     const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
     const bool active = (grp ? ntf1 : ntf0) > 0;
-    const ring::Layout lay = ring::make_layout<DT>(ntf0, ntf1, ring::ring_bytes<DT>());
+    const ring::Layout lay = ring::make_layout<DT, RB>(ntf0, ntf1, ring::ring_bytes<DT>());
 
-    ring::Loader ld;
+    ring::Loader<RB> ld;
     ld.tok_base = a.act + row0 * H * ES;
     ld.w_base[0] = a.w2 + ((int64_t)e * K + k0) * H * ES;
     ld.w_base[1] = (k0 + 128 < K) ? ld.w_base[0] + (int64_t)128 * H * ES : ld.w_base[0];
     const uint32_t row_bytes = (uint32_t)(H * ES);
     const int hb = H >> 5;
-    setup_ring_loader<DT>(
+    setup_ring_loader<DT, RB>(
         ld, lay, tid, row_bytes, ntf0, ntf1, [&](int row) { return (uint32_t)row * row_bytes; },
         a.act_scales + row0 * hb, [&](int row) { return (uint32_t)row * (uint32_t)hb; },
         a.w2_scales + (int64_t)e * K * hb,
@@ -441,14 +461,14 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     const int wrow[2] = {64 * w4, 64 * w4 + 32};
     f32x16 acc[2][4];
     zero_acc(acc);
-    const int n_slabs = (H * ES) / ring::kRB;
-    const int start = slab_rotation(n_slabs);
+    const int n_slabs = (H * ES) / RB;
+    const int start = slab_rotation<RB>(n_slabs);
     const int tok_region = grp ? lay.group1_off : 0;
     if (active) {
-        ring::main_loop<DT, NTF, false, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
+        ring::main_loop<DT, RB, NTF, false, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
         scatter_add<NTF>(acc, ri.tok + grp * kBlockRows, ri.wt + grp * kBlockRows, a.accum, K, k0 + 64 * w4, lane);
     } else {
-        ring::main_loop<DT, NTF, false, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
+        ring::main_loop<DT, RB, NTF, false, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
     }
 }
 
@@ -501,16 +521,16 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
     if (e < 0 || e >= a.E) return;
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {
-        if (skinny) down_tile_ring<DT, 1, false>(a, first, kt, e, ri, lds);
+        if (skinny) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, e, ri, lds);
         else if (ntf == 1) down_tile_wide_bf16<1>(a, first, kt, e, ri, lds);
         else if (ntf == 2) down_tile_wide_bf16<2>(a, first, kt, e, ri, lds);
         else down_tile_wide_bf16<4>(a, first, kt, e, ri, lds);
     } else {
         const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-        if (ntf == 1) down_tile_ring<DT, 1, false>(a, first, kt, e, ri, lds);
-        else if (ntf == 2) down_tile_ring<DT, 2, false>(a, first, kt, e, ri, lds);
-        else if (full) down_tile_ring<DT, 4, true>(a, first, kt, e, ri, lds);
-        else down_tile_ring<DT, 4, false>(a, first, kt, e, ri, lds);
+        if (ntf == 1) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, e, ri, lds);
+        else if (ntf == 2) down_tile_ring<DT, kPartRB, 2, false>(a, first, kt, e, ri, lds);
+        else if (full) down_tile_ring<DT, 64, 4, true>(a, first, kt, e, ri, lds);
+        else down_tile_ring<DT, kPartRB, 4, false>(a, first, kt, e, ri, lds);
     }
 }
 

@@ -1,26 +1,25 @@
-// Ring engine of the 512-thread grouped-GEMM kernels of the split pipeline, gfx950.
+// Stage-ring engine of the 512-thread grouped-GEMM kernels, gfx950: mxfp8 tiles and bf16 decode tiles
+// (the wide bf16 tiles use the unit ring of moe_ring128.h, which shares the primitives below).
 //
-// Tile: token rows x 256 weight rows.  The contraction is consumed in slabs of 64 bytes per row
-// (32 bf16 / 64 e4m3).  Slabs are copied global -> LDS by the direct-to-LDS path
-// (global_load_lds_*: no staging registers, no ds_write) into a ring of stages; all but one stage
-// are in flight while one is consumed.  One barrier per slab.
+// Tile: token rows x 256 weight rows.  The contraction is consumed in slabs of RB = 64 or 128 bytes
+// per row.  Slabs are copied global -> LDS by the direct-to-LDS path (global_load_lds_*: no staging
+// registers, no ds_write) into a ring of stages; all but one stage are in flight while one is
+// consumed.  One barrier per slab.  RB = 128 asks L2 for whole cache lines (half the requests, half
+// the barriers; a plain stream from HBM runs 8 % faster); RB = 64 has twice the stages in the same LDS.
 //
 // The ring is sized per tile.  A stage holds only the 32-row token fragments that have live rows
 // (group 0's first, then group 1's), the 256 weight rows and, for mxfp8, the scale dwords of both;
-// as many stages as fit the LDS budget are used, at most 8:
-//   two full blocks (256 token rows)       4 stages of 32 KB (+2 KB scales), 96 KB in flight per CU;
-//   one full block (128 token rows)        6 stages of 24 KB (+1.5 KB), 80 KB of weight rows in flight;
-//   a decode tile (32 live rows)           8 stages of 18 KB (+1.25 KB), 112 KB of weight rows in flight.
-// The fewer token rows a tile has, the closer it is to a pure stream of weights from HBM, and what
-// keeps HBM busy then is weight bytes in flight per CU (latency x bandwidth per CU ~ 60 KB).
+// as many stages as fit the LDS budget are used, at most 8.  The fewer token rows a tile has, the
+// closer it is to a pure stream of weights from HBM, and what keeps HBM busy then is weight bytes in
+// flight per CU.
 //
-// Stage layout: [live token rows][64 B] [256 weight rows][64 B] [scale dwords: token rows rounded up
-// to a multiple of 64, then weight rows (mxfp8)].
-// A row is 4 chunks of 16 B; chunk c of row r sits in slot c ^ ((r >> 2) & 3): the 16-byte MFMA
-// operand reads of 16 consecutive rows then cover all 64 LDS banks exactly once.  The copy engine
-// writes lane l of a wave instruction to bytes [16 l, 16 l + 16) behind a wave-uniform base, so the
-// swizzle is applied on the global side (the lane landing in slot s of row r fetches chunk
-// s ^ swz(r)).
+// Stage layout: [live token rows][RB] [256 weight rows][RB] [scale dwords: token rows rounded up to a
+// multiple of 64, then weight rows (mxfp8)].
+// A row is RB/16 chunks of 16 B; chunk c of row r sits in slot c ^ swizzle(r) (64 B: (r >> 2) & 3,
+// 128 B: (r >> 1) & 7): the 16-byte MFMA operand reads of 16 consecutive rows then cover all 64 LDS
+// banks exactly once.  The copy engine writes lane l of a wave instruction to bytes [16 l, 16 l + 16)
+// behind a wave-uniform base (one instruction = 1 KB = 1024 / RB rows), so the swizzle is applied on
+// the global side (the lane landing in slot s of row r fetches chunk s ^ swizzle(r)).
 //
 // mxfp8 scales ride along: the 4-scale dword (128 K) of every row of the tile is copied with each
 // slab into the stage's scale region, 4 bytes per lane.
@@ -36,9 +35,12 @@
 namespace pmoe {
 namespace ring {
 
-constexpr int kRB = 64;  // row bytes of a slab
-
 constexpr int kMaxStages = 8;
+
+template <int RB>
+__device__ __forceinline__ int swz(int row) {
+    return RB == 64 ? (row >> 2) & 3 : (row >> 1) & 7;
+}
 
 // Geometry of a tile's ring; every member is wave-uniform.
 struct Layout {
@@ -50,26 +52,26 @@ struct Layout {
     int stage_bytes;
     int stages;
 };
-template <int DT>
+template <int DT, int RB>
 __device__ __forceinline__ Layout make_layout(int ntf0, int ntf1, int budget) {
     Layout l;
     l.tok_rows = 32 * (ntf0 + ntf1);
-    l.group1_off = 32 * ntf0 * kRB;
-    l.w_off = l.tok_rows * kRB;
-    l.scale_off = l.w_off + kWRows * kRB;
+    l.group1_off = 32 * ntf0 * RB;
+    l.w_off = l.tok_rows * RB;
+    l.scale_off = l.w_off + kWRows * RB;
     l.scale_tok_rows = (l.tok_rows + 63) & ~63;
     const int bytes = l.scale_off + (DT == DT_FP8 ? (l.scale_tok_rows + kWRows) * 4 : 0);
     l.stage_bytes = (bytes + 255) & ~255;
     l.stages = min(kMaxStages, budget / l.stage_bytes);
     return l;
 }
-// Compile-time geometry of the tile with two full blocks (4 stages).
+// Compile-time geometry of the tile with two full blocks at RB = 64 (4 stages).
 template <int DT>
 struct FullCfg {
     static constexpr int kStages = 4;
     static constexpr int kTokRows = 256;
-    static constexpr int kWOff = kTokRows * kRB;
-    static constexpr int kScaleOff = kWOff + kWRows * kRB;
+    static constexpr int kWOff = kTokRows * 64;
+    static constexpr int kScaleOff = kWOff + kWRows * 64;
     static constexpr int kStageBytes = kScaleOff + (DT == DT_FP8 ? (kTokRows + kWRows) * 4 : 0);
 };
 // LDS the ring may use, a multiple of 1 KB (the split kernels put their row table behind it).
@@ -77,8 +79,6 @@ template <int DT>
 constexpr int ring_bytes() {
     return DT == DT_FP8 ? 156 * 1024 : 144 * 1024;
 }
-
-__device__ __forceinline__ int swz64(int row) { return (row >> 2) & 3; }
 
 __device__ __forceinline__ uint32_t lds_addr(const char *p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
@@ -102,7 +102,8 @@ __device__ __forceinline__ void wait_and_barrier() {
 }
 // Waits until at most `n` (wave-uniform, <= 30) of this wave's copies are in flight and its LDS
 // reads have returned, then joins the workgroup barrier.  The wait count is an immediate of the
-// instruction, hence the switch (at most 5 copies per stage x 6 stages behind the current one).
+// instruction, hence the switch (RB = 64: at most 5 copies per stage x 6 stages behind the current
+// one; RB = 128: 9 x 2).
 __device__ __forceinline__ void wait_and_barrier_dyn(int n) {
     switch (n) {
 #define PMOE_WB(k) case k: wait_and_barrier<k>(); break;
@@ -115,23 +116,31 @@ __device__ __forceinline__ void wait_and_barrier_dyn(int n) {
     }
 }
 
-// Per-thread description of the copies of one stage.  Every wave copies its 16 rows of both
-// 128-row halves of the weight tile.  Token rows: up to two wave instructions (wide: the wave's 16
-// rows of each group's block, if that block has live rows there; skinny: waves 0-1 copy the 32
-// rows).  Scales: at most one 4-byte-per-lane instruction per wave.
+// Per-thread description of the copies of one stage.  A 128-row block of token rows or half of the
+// weight tile takes N = RB / 64 instructions of every wave: instruction q of wave w moves rows
+// q * 8 * rpc + rpc * w .. + rpc - 1 of it (rpc = 1024 / RB rows per instruction).  Token rows of
+// fragments without live rows are not copied.  Scales: at most one 4-byte-per-lane instruction per
+// wave.
+template <int RB>
 struct Loader {
+    static constexpr int N = RB / 64;
+    static constexpr int kRowsPerCopy = 1024 / RB;
     const char *tok_base;
     const char *w_base[2];
-    uint32_t tok_off[2];
-    uint32_t w_off;
+    uint32_t tok_off[2][N];
+    uint32_t w_off[N];
     const char *sc_base;  // wave-uniform: activation scales or weight scales
     uint32_t sc_off;      // this lane's row in them
     uint32_t sc_step;     // bytes between consecutive 128-wide K tiles: 4 (row major) or 512 (blocked)
-    int tok_dst[2];       // LDS offset inside a stage of this wave's token rows; -1: nothing to copy
-    int w_dst[2];         // LDS offsets of this wave's weight rows
+    int tok_dst[2][N];    // LDS offset inside a stage of this wave's token rows; -1: nothing to copy
+    int w_dst[2][N];      // LDS offsets of this wave's weight rows
     int sc_dst;           // LDS offset of this wave's scale dwords; -1: none
     int lps;              // copy instructions this wave issues per stage
 
+    // Row inside a 128-row block that lane `lane` of wave `wave` moves with instruction q.
+    static __device__ __forceinline__ int row_of(int wave, int lane, int q) {
+        return q * 8 * kRowsPerCopy + kRowsPerCopy * wave + lane / (RB / 16);
+    }
     // The base pointers feed scalar operands of the copy instructions: pin them to scalar registers.
     __device__ __forceinline__ void make_uniform() {
         tok_base = uniform_ptr(tok_base);
@@ -139,14 +148,18 @@ struct Loader {
         w_base[1] = uniform_ptr(w_base[1]);
         sc_base = uniform_ptr(sc_base);
     }
-
     __device__ __forceinline__ void issue(char *stage, int slab) const {
-        const uint32_t koff = (uint32_t)slab * kRB;
-        if (tok_dst[0] >= 0) copy16(tok_base, tok_off[0] + koff, stage + tok_dst[0]);
-        if (tok_dst[1] >= 0) copy16(tok_base, tok_off[1] + koff, stage + tok_dst[1]);
-        copy16(w_base[0], w_off + koff, stage + w_dst[0]);
-        copy16(w_base[1], w_off + koff, stage + w_dst[1]);
-        if (sc_dst >= 0) copy4(sc_base, sc_off + (uint32_t)(slab >> 1) * sc_step, stage + sc_dst);
+        const uint32_t koff = (uint32_t)slab * RB;
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int q = 0; q < N; ++q)
+                if (tok_dst[b][q] >= 0) copy16(tok_base, tok_off[b][q] + koff, stage + tok_dst[b][q]);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int q = 0; q < N; ++q) copy16(w_base[h], w_off[q] + koff, stage + w_dst[h][q]);
+        if (sc_dst >= 0) copy4(sc_base, sc_off + (uint32_t)(RB == 64 ? slab >> 1 : slab) * sc_step, stage + sc_dst);
     }
 };
 
@@ -155,16 +168,17 @@ struct FragsBf16 {
     bf16x8 b[4];  // token fragments
 };
 
-template <int NTF>
+// Operand fragments of K sub-step j (16 bf16) of a slab: lane l holds row l % 32, chunk 2 j + l / 32.
+template <int RB, int NTF>
 __device__ __forceinline__ void fetch_bf16(FragsBf16 &fr, const char *tok, const char *wgt, const int (&wrow)[2],
                                            int lane, int j) {
-    const int r = lane & 31, half = lane >> 5, sx = (lane >> 2) & 3;
-    const int off = r * kRB + (((2 * j + half) ^ sx) << 4);
+    const int r = lane & 31, half = lane >> 5, sx = swz<RB>(r);
+    const int off = r * RB + (((2 * j + half) ^ sx) << 4);
 #pragma unroll
-    for (int f = 0; f < 2; ++f) fr.a[f] = *reinterpret_cast<const bf16x8 *>(wgt + wrow[f] * kRB + off);
+    for (int f = 0; f < 2; ++f) fr.a[f] = *reinterpret_cast<const bf16x8 *>(wgt + wrow[f] * RB + off);
 #pragma unroll
     for (int t = 0; t < 4; ++t)
-        if (t < NTF) fr.b[t] = *reinterpret_cast<const bf16x8 *>(tok + t * 32 * kRB + off);
+        if (t < NTF) fr.b[t] = *reinterpret_cast<const bf16x8 *>(tok + t * 32 * RB + off);
 }
 
 template <int NTF, bool TRANSPOSED>
@@ -181,22 +195,23 @@ __device__ __forceinline__ void mma_bf16(f32x16 (&acc)[2][4], const FragsBf16 &f
             }
 }
 
-// One e4m3 slab = one v_mfma_scale_f32_32x32x64_f8f6f4 per (weight fragment, token fragment).
-// Registers 0-3 of both lane halves form K block 0 of the slab (lanes < 32 its first 16 bytes,
-// lanes >= 32 the last 16), registers 4-7 form K block 1; the scale of block 0 is taken from lanes
-// < 32 and that of block 1 from lanes >= 32 (measured on gfx950).  `sel` = 8 * (2 * (slab & 1) +
-// lane / 32) picks this lane's scale byte out of the row's 4-scale dword.
-template <int NTF, bool TRANSPOSED>
-__device__ __forceinline__ void mma_fp8_slab(f32x16 (&acc)[2][4], const char *tok, const char *wgt,
+// 64 e4m3 of K = one v_mfma_scale_f32_32x32x64_f8f6f4 per (weight fragment, token fragment); `j` is
+// the 64-byte step inside the slab (0 for RB = 64).  Registers 0-3 of both lane halves form K block 0
+// of the step (lanes < 32 its first 16 bytes, lanes >= 32 the last 16), registers 4-7 form K block 1;
+// the scale of block 0 is taken from lanes < 32 and that of block 1 from lanes >= 32 (measured on
+// gfx950).  `sel` = 8 * (2 * (64-byte step inside its 128-wide K tile) + lane / 32) picks this lane's
+// scale byte out of the row's 4-scale dword.
+template <int RB, int NTF, bool TRANSPOSED>
+__device__ __forceinline__ void mma_fp8_step(f32x16 (&acc)[2][4], const char *tok, const char *wgt,
                                              const uint32_t *tok_sc, const uint32_t *w_sc,
-                                             const int (&wrow)[2], int lane, int sel) {
-    const int r = lane & 31, half = lane >> 5, sx = (lane >> 2) & 3;
-    const int off = r * kRB + ((half ^ sx) << 4);
+                                             const int (&wrow)[2], int lane, int j, int sel) {
+    const int r = lane & 31, half = lane >> 5, sx = swz<RB>(r);
+    const int off = r * RB + (((4 * j + half) ^ sx) << 4);
     i32x8 a[2];
     int sa[2];
 #pragma unroll
     for (int f = 0; f < 2; ++f) {
-        const char *p = wgt + wrow[f] * kRB;
+        const char *p = wgt + wrow[f] * RB;
         const i32x4 lo = *reinterpret_cast<const i32x4 *>(p + off);
         const i32x4 hi = *reinterpret_cast<const i32x4 *>(p + (off ^ 32));
         a[f] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
@@ -205,7 +220,7 @@ __device__ __forceinline__ void mma_fp8_slab(f32x16 (&acc)[2][4], const char *to
 #pragma unroll
     for (int t = 0; t < 4; ++t)
         if (t < NTF) {
-            const char *p = tok + t * 32 * kRB;
+            const char *p = tok + t * 32 * RB;
             const i32x4 lo = *reinterpret_cast<const i32x4 *>(p + off);
             const i32x4 hi = *reinterpret_cast<const i32x4 *>(p + (off ^ 32));
             const i32x8 b = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
@@ -224,16 +239,17 @@ __device__ __forceinline__ void mma_fp8_slab(f32x16 (&acc)[2][4], const char *to
 // rows): they only issue their share of the copies and join the barriers.  `tok_region` = byte
 // offset of this wave's group inside a stage's token rows.
 //
-// The slabs are visited in rotated order, starting at slab `start` (even): workgroups that run
-// side by side and share rows then ask for different cache lines at any one time instead of
-// queueing on the same ones.  The sum over K does not depend on the order.
+// The slabs are visited in rotated order, starting at slab `start` (even for RB = 64): workgroups
+// that run side by side and share rows then ask for different cache lines at any one time instead
+// of queueing on the same ones.  The sum over K does not depend on the order.
 //
-// FULL: the tile has two completely live blocks, so geometry and wait counts are compile-time
-// constants (`lay` must be that geometry); otherwise both are wave-uniform run-time values and the
-// wait count goes through a switch.
-template <int DT, int NTF, bool TRANSPOSED, bool COMPUTE, bool FULL>
-__device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader &ld, const Layout &lay, char *lds,
+// FULL (RB = 64 only): the tile has two completely live blocks, so geometry and wait counts are
+// compile-time constants (`lay` must be that geometry); otherwise both are wave-uniform run-time
+// values and the wait count goes through a switch.
+template <int DT, int RB, int NTF, bool TRANSPOSED, bool COMPUTE, bool FULL>
+__device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader<RB> &ld, const Layout &lay, char *lds,
                                           int n_slabs, const int (&wrow)[2], int lane, int tok_region, int start) {
+    static_assert(!FULL || RB == 64, "the constant geometry is the 64-byte one");
     using F = FullCfg<DT>;
     const int SB = FULL ? F::kStageBytes : lay.stage_bytes;
     const int NS = FULL ? F::kStages : lay.stages;
@@ -277,17 +293,32 @@ __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader &ld,
             const char *tok = cur + tok_region;
             const char *wgt = cur + w_off;
             if constexpr (DT == DT_BF16) {
-                // software pipeline across the barrier: the second K sub-step of a slab is held back
+                // software pipeline across the barrier: the last K sub-step of a slab is held back
                 // and issued behind the first fragment reads of the next slab
-                fetch_bf16<NTF>(fx, tok, wgt, wrow, lane, 0);
+                fetch_bf16<RB, NTF>(fx, tok, wgt, wrow, lane, 0);
                 mma_bf16<NTF, TRANSPOSED>(acc, fy);
-                fetch_bf16<NTF>(fy, tok, wgt, wrow, lane, 1);
-                mma_bf16<NTF, TRANSPOSED>(acc, fx);
+#pragma unroll
+                for (int j = 1; j < RB / 32; j += 2) {
+                    fetch_bf16<RB, NTF>(fy, tok, wgt, wrow, lane, j);
+                    mma_bf16<NTF, TRANSPOSED>(acc, fx);
+                    if (j + 1 < RB / 32) {
+                        fetch_bf16<RB, NTF>(fx, tok, wgt, wrow, lane, j + 1);
+                        mma_bf16<NTF, TRANSPOSED>(acc, fy);
+                    }
+                }
             } else {
                 const uint32_t *sc = reinterpret_cast<const uint32_t *>(cur + scale_off);
-                // start is even: the parity of kt is the parity of the slab inside its 128-wide K tile
-                mma_fp8_slab<NTF, TRANSPOSED>(acc, tok, wgt, sc + tok_region / kRB, sc + scale_tok_rows, wrow, lane,
-                                              8 * (2 * (kt & 1) + (lane >> 5)));
+                const uint32_t *tok_sc = sc + tok_region / RB, *w_sc = sc + scale_tok_rows;
+                if constexpr (RB == 64) {
+                    // start is even: the parity of kt is the parity of the slab inside its 128-wide K tile
+                    mma_fp8_step<RB, NTF, TRANSPOSED>(acc, tok, wgt, tok_sc, w_sc, wrow, lane, 0,
+                                                      8 * (2 * (kt & 1) + (lane >> 5)));
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        mma_fp8_step<RB, NTF, TRANSPOSED>(acc, tok, wgt, tok_sc, w_sc, wrow, lane, j,
+                                                          8 * (2 * j + (lane >> 5)));
+                }
             }
         }
         fill_off = cur_off;

@@ -56,21 +56,15 @@ constexpr int kPartRB = PMOE_PART_RB;      // of mxfp8 tiles with more, short of
 constexpr int kActPitchBf16 = 272;  // 128 bf16 + 16 B pad: 16-byte aligned rows, 2-way conflicts at most
 constexpr int kActPitchFp8 = 144;   // 128 e4m3 + 16 B pad
 
-// Workgroup id -> (first block, blocks, weight tile), using the live tile count read on the device.
-// Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; ids are regrouped so that
-// one XCD runs a contiguous range of logical ids, which index the work list the prologue built.
-__device__ __forceinline__ bool resolve_tile(const MoeArgs &a, int &first, int &nb, int &wt) {
-    const int n_row_tiles = min(a.n_tiles[0], a.n_blocks);
-    const int G = n_row_tiles * a.n_wtiles;
-    const int per_xcd = (G + 7) >> 3;
-    const int idx = (int)(blockIdx.x >> 3);
-    if (idx >= per_xcd) return false;
-    const int logical = (int)(blockIdx.x & 7) * per_xcd + idx;
-    if (logical >= G) return false;
-    const int2 w = a.work[logical];
+// Workgroup id -> (first block, blocks, weight tile, expert): one load from the work list, which the
+// prologue lays out by workgroup id (see emit_work); entries of workgroups without a tile are -1.
+__device__ __forceinline__ bool resolve_tile(const MoeArgs &a, int &first, int &nb, int &wt, int &e) {
+    const int2 w = a.work[blockIdx.x];
+    if (w.x < 0) return false;
     first = w.x & 0x0fffffff;
     nb = w.x >> 28;
-    wt = w.y;
+    wt = w.y & 0xffff;
+    e = w.y >> 16;
     return true;
 }
 
@@ -81,28 +75,30 @@ struct RowInfo {
     int nvalid[NG];             // per group: 1 + index of the last live row
 };
 
-// Fills RowInfo for the `nb` blocks starting at `first`; returns the largest number of 32-row
-// fragments holding live rows in any group.
-template <int NG>
-__device__ __forceinline__ int load_row_info(const MoeArgs &a, int first, int nb, RowInfo<NG> &ri) {
+// Fills tok[] and nvalid[] of RowInfo for the `nb` blocks starting at `first`; returns the largest
+// number of 32-row fragments holding live rows in any group.  The routing weight of row `tid`
+// (threads 0..255) comes back in `wt`: with NEED_WT its load is issued here and first used by the
+// caller's epilogue, so that its latency (a second dependent load behind the sorted id) overlaps the
+// K loop; the up kernel does not need it at all.
+template <int NG, bool NEED_WT>
+__device__ __forceinline__ int load_row_info(const MoeArgs &a, int first, int nb, RowInfo<NG> &ri, float &wt) {
     const int tid = threadIdx.x;
     if (tid < NG) ri.nvalid[tid] = 0;
     __syncthreads();
+    wt = 0.f;
     if (tid < kBlockRows * NG) {
         const int g = tid >> 7;
         int tok = -1;
-        float wt = 0.f;
         if (g < nb) {
             const int s = first * kBlockRows + tid;
             const int p = (s < a.sorted_num) ? a.sorted_ids[s] : -1;
             if (p >= 0) {
                 tok = p / a.top_k;
-                if (tok < a.M) wt = a.topk_w[p];
-                else tok = -1;
+                if (tok >= a.M) tok = -1;
+                else if (NEED_WT) wt = a.topk_w[p];
             }
         }
         ri.tok[tid] = tok;
-        ri.wt[tid] = wt;
         if (tok >= 0) atomicMax(&ri.nvalid[g], (tid & 127) + 1);
     }
     __syncthreads();
@@ -408,13 +404,11 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
     using L = SplitLds<DT>;
     __shared__ __attribute__((aligned(1024))) char lds[L::kTotal];
     RowInfo<2> &ri = *reinterpret_cast<RowInfo<2> *>(lds + L::kRowInfoOff);
-    int first, nb, ht;
-    if (!resolve_tile(a, first, nb, ht)) return;
-    if (first * kBlockRows >= a.ntpp[0]) return;
-    const int ntf = load_row_info<2>(a, first, nb, ri);
+    int first, nb, ht, e;
+    if (!resolve_tile(a, first, nb, ht, e)) return;
+    float wt_unused;
+    const int ntf = load_row_info<2, false>(a, first, nb, ri, wt_unused);
     if (ntf == 0) return;
-    const int e = a.expert_ids[first];
-    if (e < 0 || e >= a.E) return;
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {
         if (skinny) up_tile_ring<DT, kSkinnyRB, 1, false>(a, first, ht, e, ri, lds, nullptr);
@@ -434,7 +428,8 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
 // Down kernel of the split pipeline: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
 // full reduction over H inside the workgroup (no split-K), then w[row] * y added to accum[token].
 template <int DT, int RB, int NTF, bool FULL>
-__device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, char *lds) {
+__device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, float wt,
+                                               char *lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int grp = wave >> 2, w4 = wave & 3;
@@ -464,18 +459,19 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     const int n_slabs = (H * ES) / RB;
     const int start = slab_rotation<RB>(n_slabs);
     const int tok_region = grp ? lay.group1_off : 0;
-    if (active) {
-        ring::main_loop<DT, RB, NTF, false, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
-        scatter_add<NTF>(acc, ri.tok + grp * kBlockRows, ri.wt + grp * kBlockRows, a.accum, K, k0 + 64 * w4, lane);
-    } else {
-        ring::main_loop<DT, RB, NTF, false, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
-    }
+    if (active) ring::main_loop<DT, RB, NTF, false, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
+    else ring::main_loop<DT, RB, NTF, false, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
+    if (tid < 2 * kBlockRows) ri.wt[tid] = wt;
+    __syncthreads();
+    if (active) scatter_add<NTF>(acc, ri.tok + grp * kBlockRows, ri.wt + grp * kBlockRows, a.accum, K, k0 + 64 * w4, lane);
 }
 
-// Down kernel tile on the 128-byte ring (bf16).  The ring overwrites the row table; every thread
-// carries one of its 512 words through the K loop in a register and puts it back for the scatter.
+// Down kernel tile on the 128-byte unit ring (bf16).  The ring overwrites the row table; threads
+// 0..255 carry their row's token index (and routing weight) through the K loop in registers and put
+// them back for the scatter.
 template <int NTF>
-__device__ __forceinline__ void down_tile_wide_bf16(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, char *lds) {
+__device__ __forceinline__ void down_tile_wide_bf16(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, float wt,
+                                                    char *lds) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int grp = wave >> 2, w4 = wave & 3;
     const int K = a.K, H = a.H;
@@ -484,7 +480,7 @@ __device__ __forceinline__ void down_tile_wide_bf16(const MoeArgs &a, int first,
     const int ntf0 = __builtin_amdgcn_readfirstlane((ri.nvalid[0] + 31) >> 5);
     const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
     const bool active = (grp ? ntf1 : ntf0) > 0;
-    const int kept = tid < 2 * kBlockRows ? ri.tok[tid] : __float_as_int(ri.wt[tid - 2 * kBlockRows]);
+    const int kept_tok = tid < 2 * kBlockRows ? ri.tok[tid] : -1;
 
     const uint32_t row_bytes = (uint32_t)H * 2u;
     const char *w_lo = a.w2 + ((int64_t)e * K + k0) * H * 2;
@@ -501,8 +497,10 @@ __device__ __forceinline__ void down_tile_wide_bf16(const MoeArgs &a, int first,
     const int tok_region = grp * ring128::kGroupRegion;
     if (active) ring128::main_loop<NTF, false, true>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
     else ring128::main_loop<NTF, false, false>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
-    if (tid < 2 * kBlockRows) ri.tok[tid] = kept;
-    else ri.wt[tid - 2 * kBlockRows] = __int_as_float(kept);
+    if (tid < 2 * kBlockRows) {
+        ri.tok[tid] = kept_tok;
+        ri.wt[tid] = wt;
+    }
     __syncthreads();
     if (active) scatter_add<NTF>(acc, ri.tok + grp * kBlockRows, ri.wt + grp * kBlockRows, a.accum, K, k0 + 64 * w4, lane);
 }
@@ -512,25 +510,23 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
     using L = SplitLds<DT>;
     __shared__ __attribute__((aligned(1024))) char lds[L::kTotal];
     RowInfo<2> &ri = *reinterpret_cast<RowInfo<2> *>(lds + L::kRowInfoOff);
-    int first, nb, kt;
-    if (!resolve_tile(a, first, nb, kt)) return;
-    if (first * kBlockRows >= a.ntpp[0]) return;
-    const int ntf = load_row_info<2>(a, first, nb, ri);
+    int first, nb, kt, e;
+    if (!resolve_tile(a, first, nb, kt, e)) return;
+    float wt;  // routing weight of sorted row threadIdx.x (threads 0..255), written to the row table after the K loop
+    const int ntf = load_row_info<2, true>(a, first, nb, ri, wt);
     if (ntf == 0) return;
-    const int e = a.expert_ids[first];
-    if (e < 0 || e >= a.E) return;
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {
-        if (skinny) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, e, ri, lds);
-        else if (ntf == 1) down_tile_wide_bf16<1>(a, first, kt, e, ri, lds);
-        else if (ntf == 2) down_tile_wide_bf16<2>(a, first, kt, e, ri, lds);
-        else down_tile_wide_bf16<4>(a, first, kt, e, ri, lds);
+        if (skinny) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, e, ri, wt, lds);
+        else if (ntf == 1) down_tile_wide_bf16<1>(a, first, kt, e, ri, wt, lds);
+        else if (ntf == 2) down_tile_wide_bf16<2>(a, first, kt, e, ri, wt, lds);
+        else down_tile_wide_bf16<4>(a, first, kt, e, ri, wt, lds);
     } else {
         const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-        if (ntf == 1) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, e, ri, lds);
-        else if (ntf == 2) down_tile_ring<DT, kPartRB, 2, false>(a, first, kt, e, ri, lds);
-        else if (full) down_tile_ring<DT, 64, 4, true>(a, first, kt, e, ri, lds);
-        else down_tile_ring<DT, kPartRB, 4, false>(a, first, kt, e, ri, lds);
+        if (ntf == 1) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, e, ri, wt, lds);
+        else if (ntf == 2) down_tile_ring<DT, kPartRB, 2, false>(a, first, kt, e, ri, wt, lds);
+        else if (full) down_tile_ring<DT, 64, 4, true>(a, first, kt, e, ri, wt, lds);
+        else down_tile_ring<DT, kPartRB, 4, false>(a, first, kt, e, ri, wt, lds);
     }
 }
 
@@ -540,12 +536,18 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
 // slab by the row tiles of its expert, inside that XCD's L2.  (Walking expert by expert instead,
 // so that all row tiles of an expert always meet, measured 5 % slower on the Mixtral-like shape:
 // more workgroups then ask for the same lines at the same moment.)
-__device__ __forceinline__ void emit_work(int2 *work, int n_wt, int tile, int n_tiles, int first, int nb) {
+// Hardware hands consecutive workgroup ids to the 8 XCDs round-robin, so position `l` of the walk
+// is given to workgroup id 8 * (l mod per_xcd) + l / per_xcd: one XCD then runs a contiguous range of
+// the walk.  The entry carries everything the workgroup needs to start: (first block | blocks << 28,
+// weight tile | expert << 16).
+__device__ __forceinline__ void emit_work(int2 *work, int n_wt, int tile, int n_tiles, int first, int nb, int e) {
     constexpr int GW = 8;
+    const int per_xcd = (n_tiles * n_wt + 7) >> 3;
     for (int wt = 0; wt < n_wt; ++wt) {
         const int wg = wt / GW;
         const int gw = min(GW, n_wt - wg * GW);
-        work[wg * GW * n_tiles + tile * gw + (wt - wg * GW)] = make_int2(first | (nb << 28), wt);
+        const int l = wg * GW * n_tiles + tile * gw + (wt - wg * GW);
+        work[8 * (l % per_xcd) + l / per_xcd] = make_int2(first | (nb << 28), wt | (e << 16));
     }
 }
 
@@ -555,11 +557,14 @@ __device__ __forceinline__ void emit_work(int2 *work, int n_wt, int tile, int n_
 // tiles that writes the two walk orders.
 __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert_ids, const int32_t *ntpp,
                                                            int n_blocks, int2 *tiles, int *n_tiles,
-                                                           int2 *work_up, int n_wt_up, int2 *work_down,
-                                                           int n_wt_down, float4 *accum, int64_t n4, int do_zero) {
+                                                           int2 *work_up, int n_wt_up, int grid_up, int2 *work_down,
+                                                           int n_wt_down, int grid_down, int num_experts,
+                                                           float4 *accum, int64_t n4, int do_zero) {
     if (blockIdx.x == 0 && tiles != nullptr) {
         __shared__ int s_max[4], s_sum[4], s_carry[2];
         const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        for (int i = tid; i < grid_up; i += 256) work_up[i] = make_int2(-1, -1);
+        for (int i = tid; i < grid_down; i += 256) work_down[i] = make_int2(-1, -1);
         const int n_live = min((ntpp[0] + kBlockRows - 1) / kBlockRows, n_blocks);
         if (tid == 0) { s_carry[0] = 0; s_carry[1] = 0; }
         __syncthreads();
@@ -602,8 +607,10 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
         __syncthreads();  // tiles written above are read below by other threads
         for (int t = tid; t < nt; t += 256) {
             const int2 tl = tiles[t];
-            emit_work(work_up, n_wt_up, t, nt, tl.x, tl.y);
-            emit_work(work_down, n_wt_down, t, nt, tl.x, tl.y);
+            const int e = expert_ids[tl.x];
+            if (e < 0 || e >= num_experts) continue;  // nothing to compute for a block without an expert
+            emit_work(work_up, n_wt_up, t, nt, tl.x, tl.y, e);
+            emit_work(work_down, n_wt_down, t, nt, tl.x, tl.y, e);
         }
     }
     if (do_zero) {
@@ -694,8 +701,9 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
         const int do_zero = (mask & PMOE_PHASE_ZERO) ? 1 : 0;
         const int blocks = do_zero ? (int)std::min<int64_t>((n4 + 255) / 256, 2048) : 1;
         hipLaunchKernelGGL(moe_prologue_kernel, dim3(blocks), dim3(256), 0, s, a.expert_ids, a.ntpp, a.n_blocks,
-                           sb.tiles, sb.n_tiles, sb.work_up, a.n_wtiles,
-                           sb.work_down, n_wt_down, reinterpret_cast<float4 *>(a.accum), n4, do_zero);
+                           sb.tiles, sb.n_tiles, sb.work_up, a.n_wtiles, grid_for(a.n_blocks * a.n_wtiles),
+                           sb.work_down, n_wt_down, grid_for(a.n_blocks * n_wt_down), a.E,
+                           reinterpret_cast<float4 *>(a.accum), n4, do_zero);
     }
     if (a.n_blocks > 0) {
         a.work = sb.work_up;

@@ -31,7 +31,7 @@ import torch  # noqa: E402
 PEAK_TFLOPS = {"bf16": 2500.0, "mxfp8": 5000.0}
 PEAK_HBM_GBS = 8000.0
 
-PHASE_ZERO, PHASE_UP, PHASE_DOWN, PHASE_FINALIZE, PHASE_ALL = 1, 2, 4, 8, 15
+PHASE_PROLOGUE, PHASE_UP, PHASE_DOWN, PHASE_FINALIZE, PHASE_ALL = 1, 2, 4, 8, 15
 
 
 def build_case(cfg, device, seed=0):

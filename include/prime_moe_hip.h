@@ -59,9 +59,9 @@ int pmoe_moe_align(const int32_t *topk_ids, int32_t *sorted_token_ids, int32_t *
  * is kept so that the query takes what the call takes.
  */
 size_t pmoe_fused_moe_bf16_workspace_bytes(int M, int K, int N, int num_experts, int sorted_num,
-                                           int split);
+                                           int top_k, int split);
 size_t pmoe_fused_moe_mxfp8_workspace_bytes(int M, int K, int N, int num_experts,
-                                            int sorted_num, int split);
+                                            int sorted_num, int top_k, int split);
 
 /*
  * fused_moe_bf16 -- replaces pi::fused_moe_bf16 (torch_interface.cpp:11-34; launcher
@@ -117,10 +117,10 @@ int pmoe_quantize_mx(const void *src_bf16, void *q, void *scales, int64_t rows, 
  * kernels the two fused entry points enqueue, so a harness can time one kernel of the pipeline
  * with events around the call.  Results are only meaningful with PMOE_PHASE_ALL (the default).
  */
-#define PMOE_PHASE_ZERO 1     /* clear the fp32 accumulator */
+#define PMOE_PHASE_PROLOGUE 1 /* inversion of the sorted order (the work lists are always built) */
 #define PMOE_PHASE_UP 2       /* gate/up GEMM + SwiGLU */
-#define PMOE_PHASE_DOWN 4     /* down GEMM + routing-weight reduction */
-#define PMOE_PHASE_FINALIZE 8 /* accumulator -> bf16 `out` */
+#define PMOE_PHASE_DOWN 4     /* down GEMM */
+#define PMOE_PHASE_FINALIZE 8 /* routing-weight reduction into bf16 `out` */
 #define PMOE_PHASE_ALL 15
 void pmoe_set_phase_mask(int mask);
 

@@ -5,14 +5,16 @@
 // prime_moe/csrc/kernels/fused_moe_bf16_kernel.cu:21-733 and fused_moe_mxfp8_kernel.cu:56-866.
 //
 // Pipeline of one call (all on the caller's stream):
-//   prologue (zero the fp32 accumulator, pair blocks into row tiles, build the two work lists)
+//   prologue (pair blocks into row tiles, build the two work lists, invert the sorted order:
+//             pair id -> sorted row)
 //   -> up kernel (gate/up GEMM + SwiGLU, activation tile -> workspace)
-//   -> down kernel (fp32 atomics into the accumulator, one addend per routed pair)
-//   -> finalize: split != 0: out = bf16(accum); split == 0: out = bf16(float(out) + accum), the
-//      reference's accumulate-into-out contract of its single-kernel path.
+//   -> down kernel (y[sorted row, :K] = act . W2[e]^T, bf16, -> workspace)
+//   -> finalize: out[t] = bf16(sum over the token's pairs p of w[p] * y[row(p)]), fp32 sum in pair
+//      order; split == 0: added to `out` (the reference's accumulate-into-out contract of its
+//      single-kernel path), split != 0: `out` overwritten.
 // Both values of `split` run the same kernels: on this hardware the two-kernel pipeline is the faster
-// one at every shape, so `split` only selects what finalize does with `out`.
-// The top-k reduction is exact in fp32 up to summation order; `out` is rounded to bf16 once.
+// one at every shape, so `split` only selects what finalize does with `out`.  No atomics: the result
+// is a pure function of the inputs.
 #include <algorithm>
 
 #include "moe_ring.h"
@@ -35,7 +37,8 @@ struct MoeArgs {
     const float *topk_w;
     char *act;            // (sorted_num, H) activation workspace (split pipeline)
     uint8_t *act_scales;  // (sorted_num, H/32) e8m0, row major (mxfp8 split pipeline)
-    float *accum;         // (M, K) fp32 accumulator
+    char *y;              // (sorted_num, K) bf16: down-projected rows, before the routing weights
+    int32_t *inv;         // (M * top_k): sorted row of each pair id (validated against sorted_ids when read)
     const int2 *tiles;    // row tiles built by the prologue: (first block, number of blocks 1..2)
     const int *n_tiles;   // number of row tiles
     const int2 *work;     // this kernel's tile order: (first block | blocks << 28, weight tile)
@@ -71,21 +74,16 @@ __device__ __forceinline__ bool resolve_tile(const MoeArgs &a, int &first, int &
 template <int NG>
 struct RowInfo {
     int tok[kBlockRows * NG];   // token index of each sorted row, -1 for padding / dropped rows
-    float wt[kBlockRows * NG];  // routing weight of the row's pair
     int nvalid[NG];             // per group: 1 + index of the last live row
 };
 
-// Fills tok[] and nvalid[] of RowInfo for the `nb` blocks starting at `first`; returns the largest
-// number of 32-row fragments holding live rows in any group.  The routing weight of row `tid`
-// (threads 0..255) comes back in `wt`: with NEED_WT its load is issued here and first used by the
-// caller's epilogue, so that its latency (a second dependent load behind the sorted id) overlaps the
-// K loop; the up kernel does not need it at all.
-template <int NG, bool NEED_WT>
-__device__ __forceinline__ int load_row_info(const MoeArgs &a, int first, int nb, RowInfo<NG> &ri, float &wt) {
+// Fills RowInfo for the `nb` blocks starting at `first`; returns the largest number of 32-row
+// fragments holding live rows in any group.
+template <int NG>
+__device__ __forceinline__ int load_row_info(const MoeArgs &a, int first, int nb, RowInfo<NG> &ri) {
     const int tid = threadIdx.x;
     if (tid < NG) ri.nvalid[tid] = 0;
     __syncthreads();
-    wt = 0.f;
     if (tid < kBlockRows * NG) {
         const int g = tid >> 7;
         int tok = -1;
@@ -95,7 +93,6 @@ __device__ __forceinline__ int load_row_info(const MoeArgs &a, int first, int nb
             if (p >= 0) {
                 tok = p / a.top_k;
                 if (tok >= a.M) tok = -1;
-                else if (NEED_WT) wt = a.topk_w[p];
             }
         }
         ri.tok[tid] = tok;
@@ -117,30 +114,62 @@ __device__ __forceinline__ void zero_acc(f32x16 (&acc)[2][4]) {
             for (int i = 0; i < 16; ++i) acc[f][t][i] = 0.f;
 }
 
-// Adds w[row] * acc into accum[token, col] for the live rows of a group's block.  Accumulator
-// layout (tokens on the MFMA M side): register i of lane l = row 32t + 8(i/4) + 4(l/32) + i%4,
-// column col0 + 32f + l%32, so one instruction adds two 128-byte runs.
+// Epilogue of the down GEMM.  Weight rows (output columns) sit on the MFMA M side: register i of lane
+// l = output column 64 w4 + 32 f + 8(i/4) + 4(l/32) + i%4 of sorted row 32 t + l%32.  The group's
+// 128 x 256 tile is rounded to bf16 into `tile` (row pitch kYPitch) ...
+constexpr int kYPitch = 528;  // 256 bf16 + 16 B pad
 template <int NTF>
-__device__ __forceinline__ void scatter_add(const f32x16 (&acc)[2][4], const int *row_tok,
-                                            const float *row_wt, float *accum, int K, int col0, int lane) {
-    const int half = lane >> 5;
-    const int c = lane & 31;
+__device__ __forceinline__ void y_epilogue(const f32x16 (&acc)[2][4], char *tile, int w4, int lane) {
+    const int r = lane & 31, half = lane >> 5;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         if (t < NTF) {
+            const int row = 32 * t + r;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int row = 32 * t + 8 * (i >> 2) + 4 * half + (i & 3);
-                const int tok = row_tok[row];
-                const float w = row_wt[row];
-                if (tok >= 0) {
+            for (int f = 0; f < 2; ++f)
 #pragma unroll
-                    for (int f = 0; f < 2; ++f) {
-                        const int col = col0 + 32 * f + c;
-                        if (col < K) unsafeAtomicAdd(accum + (int64_t)tok * K + col, w * acc[f][t][i]);
-                    }
+                for (int g = 0; g < 4; ++g) {
+                    const int col = 64 * w4 + 32 * f + 8 * g + 4 * half;
+                    uint2 pk;
+                    pk.x = pack2_bf16(acc[f][t][4 * g], acc[f][t][4 * g + 1]);
+                    pk.y = pack2_bf16(acc[f][t][4 * g + 2], acc[f][t][4 * g + 3]);
+                    *reinterpret_cast<uint2 *>(tile + row * kYPitch + col * 2) = pk;
                 }
+        }
+    }
+}
+// Tiles with a single live fragment skip the detour through LDS: every lane stores its 8-byte runs
+// straight to y (32 rows x 16 KB per tile at most; a barrier and an LDS round trip cost more).
+__device__ __forceinline__ void store_y_direct(const MoeArgs &a, const f32x16 (&acc)[2][4], int64_t row0, int k0,
+                                               int n_rows, int w4, int lane) {
+    const int r = lane & 31, half = lane >> 5;
+    if (r >= n_rows) return;
+    char *dst = a.y + ((row0 + r) * a.K + k0) * 2;
+#pragma unroll
+    for (int f = 0; f < 2; ++f)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int col = 64 * w4 + 32 * f + 8 * g + 4 * half;
+            if (k0 + col < a.K) {
+                uint2 pk;
+                pk.x = pack2_bf16(acc[f][0][4 * g], acc[f][0][4 * g + 1]);
+                pk.y = pack2_bf16(acc[f][0][4 * g + 2], acc[f][0][4 * g + 3]);
+                *reinterpret_cast<uint2 *>(dst + col * 2) = pk;
             }
+        }
+}
+// ... and its first n_rows rows are copied to y rows row0.., columns [k0, k0 + 256) (the last
+// tile of a K that is not a multiple of 256 has 128 columns); gt = thread index inside the group.
+__device__ __forceinline__ void store_y_tile(const MoeArgs &a, const char *tile, int64_t row0, int k0, int n_rows, int gt) {
+    const int K = a.K;
+    const int c = gt & 31;
+    if (k0 + 8 * c >= K) return;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int row = (gt >> 5) + 8 * i;
+        if (row < n_rows) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kYPitch + c * 16);
+            *reinterpret_cast<uint4 *>(a.y + ((row0 + row) * K + k0) * 2 + c * 16) = v;
         }
     }
 }
@@ -406,8 +435,7 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
     RowInfo<2> &ri = *reinterpret_cast<RowInfo<2> *>(lds + L::kRowInfoOff);
     int first, nb, ht, e;
     if (!resolve_tile(a, first, nb, ht, e)) return;
-    float wt_unused;
-    const int ntf = load_row_info<2, false>(a, first, nb, ri, wt_unused);
+    const int ntf = load_row_info<2>(a, first, nb, ri);
     if (ntf == 0) return;
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {
@@ -428,17 +456,18 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
 // Down kernel of the split pipeline: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
 // full reduction over H inside the workgroup (no split-K), then w[row] * y added to accum[token].
 template <int DT, int RB, int NTF, bool FULL>
-__device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, float wt,
-                                               char *lds) {
+__device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, char *lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int grp = wave >> 2, w4 = wave & 3;
+    const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
     const int K = a.K, H = a.H;
     const int k0 = kt * kWRows;
     const int64_t row0 = (int64_t)first * kBlockRows;
     const int ntf0 = __builtin_amdgcn_readfirstlane((ri.nvalid[0] + 31) >> 5);
     const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
-    const bool active = (grp ? ntf1 : ntf0) > 0;
+    const int my_ntf = grp ? ntf1 : ntf0;
+    const int my_rows = ri.nvalid[grp];  // rows past the last live one are never read back
+    const bool active = my_ntf > 0;
     const ring::Layout lay = ring::make_layout<DT, RB>(ntf0, ntf1, ring::ring_bytes<DT>());
 
     ring::Loader<RB> ld;
@@ -459,28 +488,32 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     const int n_slabs = (H * ES) / RB;
     const int start = slab_rotation<RB>(n_slabs);
     const int tok_region = grp ? lay.group1_off : 0;
-    if (active) ring::main_loop<DT, RB, NTF, false, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
-    else ring::main_loop<DT, RB, NTF, false, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
-    if (tid < 2 * kBlockRows) ri.wt[tid] = wt;
-    __syncthreads();
-    if (active) scatter_add<NTF>(acc, ri.tok + grp * kBlockRows, ri.wt + grp * kBlockRows, a.accum, K, k0 + 64 * w4, lane);
+    if (active) ring::main_loop<DT, RB, NTF, true, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
+    else ring::main_loop<DT, RB, NTF, true, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
+    // the ring is free (main_loop ends with a barrier): reuse it for the two 128 x 256 output tiles
+    if constexpr (NTF == 1) {
+        if (active) store_y_direct(a, acc, row0 + grp * kBlockRows, k0, my_rows, w4, lane);
+    } else {
+        char *tile = lds + grp * (kBlockRows * kYPitch);
+        if (active) y_epilogue<NTF>(acc, tile, w4, lane);
+        __syncthreads();
+        if (active) store_y_tile(a, tile, row0 + grp * kBlockRows, k0, my_rows, gt);
+    }
 }
 
-// Down kernel tile on the 128-byte unit ring (bf16).  The ring overwrites the row table; threads
-// 0..255 carry their row's token index (and routing weight) through the K loop in registers and put
-// them back for the scatter.
+// Down kernel tile on the 128-byte unit ring (bf16).
 template <int NTF>
-__device__ __forceinline__ void down_tile_wide_bf16(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, float wt,
-                                                    char *lds) {
+__device__ __forceinline__ void down_tile_wide_bf16(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, char *lds) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int grp = wave >> 2, w4 = wave & 3;
+    const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
     const int K = a.K, H = a.H;
     const int k0 = kt * kWRows;
     const int64_t row0 = (int64_t)first * kBlockRows;
     const int ntf0 = __builtin_amdgcn_readfirstlane((ri.nvalid[0] + 31) >> 5);
     const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
-    const bool active = (grp ? ntf1 : ntf0) > 0;
-    const int kept_tok = tid < 2 * kBlockRows ? ri.tok[tid] : -1;
+    const int my_ntf = grp ? ntf1 : ntf0;
+    const int my_rows = ri.nvalid[grp];  // read before the ring overwrites the row table
+    const bool active = my_ntf > 0;
 
     const uint32_t row_bytes = (uint32_t)H * 2u;
     const char *w_lo = a.w2 + ((int64_t)e * K + k0) * H * 2;
@@ -495,14 +528,16 @@ __device__ __forceinline__ void down_tile_wide_bf16(const MoeArgs &a, int first,
     const int n_slabs = (int)(row_bytes / ring128::kRB);
     const int start = slab_rotation128(n_slabs);
     const int tok_region = grp * ring128::kGroupRegion;
-    if (active) ring128::main_loop<NTF, false, true>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
-    else ring128::main_loop<NTF, false, false>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
-    if (tid < 2 * kBlockRows) {
-        ri.tok[tid] = kept_tok;
-        ri.wt[tid] = wt;
+    if (active) ring128::main_loop<NTF, true, true>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
+    else ring128::main_loop<NTF, true, false>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
+    if constexpr (NTF == 1) {
+        if (active) store_y_direct(a, acc, row0 + grp * kBlockRows, k0, my_rows, w4, lane);
+    } else {
+        char *tile = lds + grp * (kBlockRows * kYPitch);
+        if (active) y_epilogue<NTF>(acc, tile, w4, lane);
+        __syncthreads();
+        if (active) store_y_tile(a, tile, row0 + grp * kBlockRows, k0, my_rows, gt);
     }
-    __syncthreads();
-    if (active) scatter_add<NTF>(acc, ri.tok + grp * kBlockRows, ri.wt + grp * kBlockRows, a.accum, K, k0 + 64 * w4, lane);
 }
 
 template <int DT>
@@ -512,21 +547,20 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
     RowInfo<2> &ri = *reinterpret_cast<RowInfo<2> *>(lds + L::kRowInfoOff);
     int first, nb, kt, e;
     if (!resolve_tile(a, first, nb, kt, e)) return;
-    float wt;  // routing weight of sorted row threadIdx.x (threads 0..255), written to the row table after the K loop
-    const int ntf = load_row_info<2, true>(a, first, nb, ri, wt);
+    const int ntf = load_row_info<2>(a, first, nb, ri);
     if (ntf == 0) return;
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {
-        if (skinny) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, e, ri, wt, lds);
-        else if (ntf == 1) down_tile_wide_bf16<1>(a, first, kt, e, ri, wt, lds);
-        else if (ntf == 2) down_tile_wide_bf16<2>(a, first, kt, e, ri, wt, lds);
-        else down_tile_wide_bf16<4>(a, first, kt, e, ri, wt, lds);
+        if (skinny) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, e, ri, lds);
+        else if (ntf == 1) down_tile_wide_bf16<1>(a, first, kt, e, ri, lds);
+        else if (ntf == 2) down_tile_wide_bf16<2>(a, first, kt, e, ri, lds);
+        else down_tile_wide_bf16<4>(a, first, kt, e, ri, lds);
     } else {
         const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-        if (ntf == 1) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, e, ri, wt, lds);
-        else if (ntf == 2) down_tile_ring<DT, kPartRB, 2, false>(a, first, kt, e, ri, wt, lds);
-        else if (full) down_tile_ring<DT, 64, 4, true>(a, first, kt, e, ri, wt, lds);
-        else down_tile_ring<DT, kPartRB, 4, false>(a, first, kt, e, ri, wt, lds);
+        if (ntf == 1) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, e, ri, lds);
+        else if (ntf == 2) down_tile_ring<DT, kPartRB, 2, false>(a, first, kt, e, ri, lds);
+        else if (full) down_tile_ring<DT, 64, 4, true>(a, first, kt, e, ri, lds);
+        else down_tile_ring<DT, kPartRB, 4, false>(a, first, kt, e, ri, lds);
     }
 }
 
@@ -551,15 +585,17 @@ __device__ __forceinline__ void emit_work(int2 *work, int n_wt, int tile, int n_
     }
 }
 
-// Prologue of every call: clears the fp32 accumulator and (workgroup 0) builds the row tiles and
-// work lists of the two-group kernels: consecutive blocks of one expert are paired, an expert's odd
-// last block stays single.  One pass of block-wide scans per 256 blocks, then one pass over the
-// tiles that writes the two walk orders.
+// Prologue of every call.  Workgroup 0 builds the row tiles and work lists of the two-group kernels:
+// consecutive blocks of one expert are paired, an expert's odd last block stays single (one pass of
+// block-wide scans per 256 blocks, then one pass over the tiles that writes the two walk orders).
+// All workgroups invert the sorted order: inv[pair id] = sorted row.  Entries of pairs that are not
+// in the schedule keep whatever the buffer held; the reader validates an entry against sorted_ids.
 __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert_ids, const int32_t *ntpp,
                                                            int n_blocks, int2 *tiles, int *n_tiles,
                                                            int2 *work_up, int n_wt_up, int grid_up, int2 *work_down,
                                                            int n_wt_down, int grid_down, int num_experts,
-                                                           float4 *accum, int64_t n4, int do_zero) {
+                                                           const int32_t *sorted_ids, int sorted_num, int32_t *inv,
+                                                           int n_pairs, int do_invert) {
     if (blockIdx.x == 0 && tiles != nullptr) {
         __shared__ int s_max[4], s_sum[4], s_carry[2];
         const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -613,23 +649,46 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
             emit_work(work_down, n_wt_down, t, nt, tl.x, tl.y, e);
         }
     }
-    if (do_zero) {
-        const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-        for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride)
-            accum[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (do_invert) {
+        const int n_rows = min(ntpp[0], sorted_num);
+        const int stride = (int)(gridDim.x * blockDim.x);
+        for (int s = (int)(blockIdx.x * blockDim.x + threadIdx.x); s < n_rows; s += stride) {
+            const int p = sorted_ids[s];
+            if (p >= 0 && p < n_pairs) inv[p] = s;
+        }
     }
 }
 
-// out = bf16(accum)  (ACCUMULATE: out = bf16(float(out) + accum)); 8 elements per thread step.
+// out[t, 8 columns] = bf16(sum over the token's top_k pairs p, in pair order, of w[p] * y[row(p)])
+// (ACCUMULATE: added to what `out` holds).  row(p) = inv[p] if that row really holds p, else the
+// pair was dropped by the schedule and contributes nothing.  One thread per (token, 8 columns).
 template <bool ACCUMULATE>
-__global__ __launch_bounds__(256) void finalize_kernel(const float4 *acc, uint4 *out, int64_t n8) {
+__global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int32_t *inv, const int32_t *sorted_ids,
+                                                       const int32_t *ntpp, int sorted_num, const float *topk_w,
+                                                       int top_k, int M, int K, uint4 *out) {
+    const int k8 = K >> 3;
+    const int64_t total = (int64_t)M * k8;
+    const int n_rows = min(ntpp[0], sorted_num);
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += stride) {
-        float4 lo = acc[2 * i], hi = acc[2 * i + 1];
-        float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-        uint32_t o[4] = {0, 0, 0, 0};
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int t = (int)(i / k8), c = (int)(i - (int64_t)t * k8);
+        float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int r = 0; r < top_k; ++r) {
+            const int p = t * top_k + r;
+            const int row = inv[p];
+            if (row < 0 || row >= n_rows || sorted_ids[row] != p) continue;
+            const float w = topk_w[p];
+            const uint4 q = *reinterpret_cast<const uint4 *>(y + ((int64_t)row * K + 8 * c) * 2);
+            const uint32_t u[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[2 * j] += w * bf16_bits_to_f32(u[j] & 0xffffu);
+                v[2 * j + 1] += w * bf16_bits_to_f32(u[j] >> 16);
+            }
+        }
+        uint32_t o[4];
         if constexpr (ACCUMULATE) {
-            uint4 prev = out[i];
+            const uint4 prev = out[i];
             o[0] = prev.x; o[1] = prev.y; o[2] = prev.z; o[3] = prev.w;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -646,10 +705,10 @@ __global__ __launch_bounds__(256) void finalize_kernel(const float4 *acc, uint4 
 // ------------------------------------------------------------------------------------------ host
 
 struct WorkspaceLayout {
-    size_t n_tiles_off, tiles_off, work_up_off, work_down_off, accum_off, act_off, act_scales_off, total;
+    size_t n_tiles_off, tiles_off, work_up_off, work_down_off, inv_off, y_off, act_off, act_scales_off, total;
 };
 
-static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_num) {
+static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_num, int top_k) {
     WorkspaceLayout l{};
     const size_t H = (size_t)N / 2;
     const size_t rows = align_up((size_t)sorted_num, kBlockRows);
@@ -663,8 +722,10 @@ static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_
     off = align_up(off + blocks * (H / 128) * sizeof(int2), 256);
     l.work_down_off = off;
     off = align_up(off + blocks * (((size_t)K + kWRows - 1) / kWRows) * sizeof(int2), 256);
-    l.accum_off = off;
-    off = align_up(off + (size_t)M * K * sizeof(float), 256);
+    l.inv_off = off;
+    off = align_up(off + (size_t)M * (size_t)std::max(top_k, 1) * sizeof(int32_t), 256);
+    l.y_off = off;
+    off = align_up(off + rows * K * 2, 256);
     l.act_off = off;
     off = align_up(off + rows * H * (dt == DT_BF16 ? 2 : 1), 256);
     l.act_scales_off = off;
@@ -696,14 +757,13 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
     a.n_tiles = sb.n_tiles;
     const int n_wt_down = (a.K + kWRows - 1) / kWRows;
     {
-        // the tile lists are needed by the two-group kernels even when the clear is masked off
-        const int64_t n4 = n_out / 4;
-        const int do_zero = (mask & PMOE_PHASE_ZERO) ? 1 : 0;
-        const int blocks = do_zero ? (int)std::min<int64_t>((n4 + 255) / 256, 2048) : 1;
+        // the work lists are needed by the two kernels even when the rest of the prologue is masked off
+        const int do_invert = (mask & PMOE_PHASE_PROLOGUE) ? 1 : 0;
+        const int blocks = do_invert ? std::max(1, std::min((a.sorted_num + 255) / 256, 1024)) : 1;
         hipLaunchKernelGGL(moe_prologue_kernel, dim3(blocks), dim3(256), 0, s, a.expert_ids, a.ntpp, a.n_blocks,
                            sb.tiles, sb.n_tiles, sb.work_up, a.n_wtiles, grid_for(a.n_blocks * a.n_wtiles),
                            sb.work_down, n_wt_down, grid_for(a.n_blocks * n_wt_down), a.E,
-                           reinterpret_cast<float4 *>(a.accum), n4, do_zero);
+                           a.sorted_ids, a.sorted_num, a.inv, a.M * a.top_k, do_invert);
     }
     if (a.n_blocks > 0) {
         a.work = sb.work_up;
@@ -717,13 +777,13 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
     }
     if (mask & PMOE_PHASE_FINALIZE) {
         const int64_t n8 = n_out / 8;
-        const int blocks = (int)std::min<int64_t>((n8 + 255) / 256, 2048);
+        const int blocks = (int)std::min<int64_t>((n8 + 255) / 256, 8192);
         if (split)
-            hipLaunchKernelGGL(finalize_kernel<false>, dim3(blocks), dim3(256), 0, s,
-                               reinterpret_cast<const float4 *>(a.accum), reinterpret_cast<uint4 *>(out), n8);
+            hipLaunchKernelGGL(finalize_kernel<false>, dim3(blocks), dim3(256), 0, s, a.y, a.inv, a.sorted_ids, a.ntpp,
+                               a.sorted_num, a.topk_w, a.top_k, a.M, a.K, reinterpret_cast<uint4 *>(out));
         else
-            hipLaunchKernelGGL(finalize_kernel<true>, dim3(blocks), dim3(256), 0, s,
-                               reinterpret_cast<const float4 *>(a.accum), reinterpret_cast<uint4 *>(out), n8);
+            hipLaunchKernelGGL(finalize_kernel<true>, dim3(blocks), dim3(256), 0, s, a.y, a.inv, a.sorted_ids, a.ntpp,
+                               a.sorted_num, a.topk_w, a.top_k, a.M, a.K, reinterpret_cast<uint4 *>(out));
     }
     return check_launch("fused_moe launch");
 }
@@ -744,17 +804,17 @@ using namespace pmoe;
 extern "C" void pmoe_set_phase_mask(int mask) { g_phase_mask = mask; }
 
 extern "C" size_t pmoe_fused_moe_bf16_workspace_bytes(int M, int K, int N, int num_experts,
-                                                      int sorted_num, int split) {
+                                                      int sorted_num, int top_k, int split) {
     (void)num_experts;
     if (M <= 0 || K <= 0 || N <= 0 || sorted_num < 0) return 0;
-    return workspace_layout(DT_BF16, M, K, N, sorted_num).total;
+    return workspace_layout(DT_BF16, M, K, N, sorted_num, top_k).total;
 }
 
 extern "C" size_t pmoe_fused_moe_mxfp8_workspace_bytes(int M, int K, int N, int num_experts,
-                                                       int sorted_num, int split) {
+                                                       int sorted_num, int top_k, int split) {
     (void)num_experts;
     if (M <= 0 || K <= 0 || N <= 0 || sorted_num < 0) return 0;
-    return workspace_layout(DT_FP8, M, K, N, sorted_num).total;
+    return workspace_layout(DT_FP8, M, K, N, sorted_num, top_k).total;
 }
 
 static int check_tuning(const char *op, int block_m, int block_n, int warp_n, int stages,
@@ -781,7 +841,7 @@ extern "C" int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2,
     PMOE_REQUIRE(top_k > 0 && num_experts > 0 && sorted_num >= 0, "fused_moe_bf16: bad top_k / num_experts / sorted_num");
     PMOE_REQUIRE(x && w && w2 && out && sorted_token_ids && expert_idxs && num_tokens_post_padded && topk_weights,
                  "fused_moe_bf16: null pointer");
-    const WorkspaceLayout l = workspace_layout(DT_BF16, M, K, N, sorted_num);
+    const WorkspaceLayout l = workspace_layout(DT_BF16, M, K, N, sorted_num, top_k);
     PMOE_REQUIRE(workspace && workspace_bytes >= l.total, "fused_moe_bf16: workspace of %zu bytes needed, got %zu", l.total, workspace_bytes);
     PMOE_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, "fused_moe_bf16: workspace must be 256-byte aligned");
     MoeArgs a{};
@@ -793,7 +853,8 @@ extern "C" int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2,
     a.ntpp = num_tokens_post_padded;
     a.topk_w = topk_weights;
     char *ws = static_cast<char *>(workspace);
-    a.accum = reinterpret_cast<float *>(ws + l.accum_off);
+    a.y = ws + l.y_off;
+    a.inv = reinterpret_cast<int32_t *>(ws + l.inv_off);
     a.act = ws + l.act_off;
     a.top_k = top_k; a.M = M; a.K = K; a.N = N; a.H = N / 2; a.E = num_experts; a.sorted_num = sorted_num;
     return launch_pipeline<DT_BF16>(a, sched_buffers(ws, l), out, split, static_cast<hipStream_t>(stream));
@@ -816,7 +877,7 @@ extern "C" int pmoe_fused_moe_mxfp8(const void *x, const void *x_scales, const v
     PMOE_REQUIRE(x && x_scales && w && w_scales && w2 && w2_scales && out && sorted_token_ids && expert_idxs &&
                      num_tokens_post_padded && topk_weights,
                  "fused_moe_mxfp8: null pointer");
-    const WorkspaceLayout l = workspace_layout(DT_FP8, M, K, N, sorted_num);
+    const WorkspaceLayout l = workspace_layout(DT_FP8, M, K, N, sorted_num, top_k);
     PMOE_REQUIRE(workspace && workspace_bytes >= l.total, "fused_moe_mxfp8: workspace of %zu bytes needed, got %zu", l.total, workspace_bytes);
     PMOE_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, "fused_moe_mxfp8: workspace must be 256-byte aligned");
     MoeArgs a{};
@@ -831,7 +892,8 @@ extern "C" int pmoe_fused_moe_mxfp8(const void *x, const void *x_scales, const v
     a.ntpp = num_tokens_post_padded;
     a.topk_w = topk_weights;
     char *ws = static_cast<char *>(workspace);
-    a.accum = reinterpret_cast<float *>(ws + l.accum_off);
+    a.y = ws + l.y_off;
+    a.inv = reinterpret_cast<int32_t *>(ws + l.inv_off);
     a.act = ws + l.act_off;
     a.act_scales = reinterpret_cast<uint8_t *>(ws + l.act_scales_off);
     a.top_k = top_k; a.M = M; a.K = K; a.N = N; a.H = N / 2; a.E = num_experts; a.sorted_num = sorted_num;

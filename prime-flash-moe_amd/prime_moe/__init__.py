@@ -135,7 +135,7 @@ def _fused_moe_bf16_impl(x, w, w2, sorted_token_ids, expert_ids, num_tokens_post
     S = sorted_token_ids.size(0)
     dev = x.device
     with torch.cuda.device(dev):
-        nbytes = lib.pmoe_fused_moe_bf16_workspace_bytes(M, K, N, E, S, int(split))
+        nbytes = lib.pmoe_fused_moe_bf16_workspace_bytes(M, K, N, E, S, top_k, int(split))
         ws = _workspace(nbytes, dev)
         _native.check(lib.pmoe_fused_moe_bf16(
             x.data_ptr(), w.data_ptr(), w2.data_ptr(), out.data_ptr(), sorted_token_ids.data_ptr(),
@@ -201,7 +201,7 @@ def _fused_moe_mxfp8_impl(x, x_scales, w, w_scales, w2, w2_scales, sorted_token_
     S = sorted_token_ids.size(0)
     dev = x.device
     with torch.cuda.device(dev):
-        nbytes = lib.pmoe_fused_moe_mxfp8_workspace_bytes(M, K, N, E, S, int(split))
+        nbytes = lib.pmoe_fused_moe_mxfp8_workspace_bytes(M, K, N, E, S, top_k, int(split))
         ws = _workspace(nbytes, dev)
         _native.check(lib.pmoe_fused_moe_mxfp8(
             x.data_ptr(), x_scales.data_ptr(), w.data_ptr(), w_scales.data_ptr(), w2.data_ptr(),

@@ -135,3 +135,18 @@ def test_validation_errors(device):
         call(x=x.t().contiguous().t())
     with pytest.raises(RuntimeError):
         call(x=x[:, :192].contiguous())
+
+
+def test_result_is_bitwise_reproducible(device):
+    """No atomics anywhere in the pipeline: two calls on the same inputs agree bit for bit."""
+    import prime_moe
+    g, x, w1, w2 = _inputs(300, 512, 8, 512, device, seed=5)
+    ids, wts = reference_routing(300, 8, 4, device, g)
+    sched = torch.ops.prime_moe.moe_align(ids, 8, 128, 1)
+    outs = []
+    for _ in range(3):
+        out = torch.empty((300, 512), dtype=torch.bfloat16, device=device)
+        prime_moe.fused_moe_bf16(x, w1, w2, *sched, wts, out, 4, 128, 64, 4, 2, 1, 1, True)
+        outs.append(out)
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])

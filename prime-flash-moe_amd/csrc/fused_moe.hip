@@ -36,7 +36,11 @@ struct MoeArgs {
     const int32_t *ntpp;
     const float *topk_w;
     char *act;            // (sorted_num, H) activation workspace (split pipeline)
-    uint8_t *act_scales;  // (sorted_num, H/32) e8m0, row major (mxfp8 split pipeline)
+    // e8m0 scales of the token-side operands of the two mxfp8 GEMMs, as the loaders want them: one
+    // dword (4 scales = 128 contraction elements) per row, [sorted block][128-wide K tile][row in block],
+    // so that the 64 lanes of a copy instruction read 256 contiguous bytes.
+    uint32_t *xs_tiled;   // scales of the gathered x rows (written by the prologue from x_scales)
+    uint32_t *act_scales; // scales of the activation (written by the up kernel's epilogue)
     char *y;              // (sorted_num, K) bf16: down-projected rows, before the routing weights
     int32_t *inv;         // (M * top_k): sorted row of each pair id (validated against sorted_ids when read)
     const int2 *tiles;    // row tiles built by the prologue: (first block, number of blocks 1..2)
@@ -248,7 +252,7 @@ __device__ __forceinline__ void store_act_tile(const MoeArgs &a, const char *til
             }
         }
         if (gt < 32 * ntf)
-            *reinterpret_cast<uint32_t *>(a.act_scales + (row0 + gt) * (H >> 5) + (h0 >> 7) * 4) = sc_tile[gt];
+            a.act_scales[((row0 >> 7) * (H >> 7) + (h0 >> 7)) * kBlockRows + gt] = sc_tile[gt];
     }
 }
 
@@ -259,7 +263,8 @@ __device__ __forceinline__ void store_act_tile(const MoeArgs &a, const char *til
 // Common set-up of the stage-ring loader.  Token rows: `tok_row_off(row)` gives the byte offset of
 // tile row `row` (0..255: block 0, then block 1) in `tok_base`; weight rows: the tile's two 128-row
 // halves start at w_base[0/1] with `w_pitch` bytes per row.  Scales (mxfp8): `tok_sc_off(row)` /
-// `w_sc_off(row)` are the byte offsets of the row's first 4-scale dword.  Only the live 32-row
+// `w_sc_off(row)` are the byte offsets of the row's first 4-scale dword; the dword of the next 128-wide
+// K tile lies 512 bytes on in both (blocked weight scales, tiled token-side scales).  Only the live 32-row
 // fragments of the two blocks (ntf0, ntf1 of them) are copied; they are packed one after the other in
 // the stage (see ring::Layout).
 template <int DT, int RB, typename TokOff, typename TokScOff, typename WScOff>
@@ -306,7 +311,7 @@ __device__ __forceinline__ void setup_ring_loader(ring::Loader<RB> &ld, const ri
             const int row = c < 32 * ntf0 ? c : kBlockRows + c - 32 * ntf0;
             ld.sc_base = reinterpret_cast<const char *>(tok_sc_base);
             ld.sc_off = tok_sc_off(row);
-            ld.sc_step = 4u;
+            ld.sc_step = 512u;
             ld.sc_dst = lay.scale_off + 64 * wave * 4;
         }
     }
@@ -351,11 +356,12 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
     ld.w_base[0] = a.w1 + ((int64_t)e * N + h0) * K * ES;
     ld.w_base[1] = ld.w_base[0] + (int64_t)H * K * ES;
     const uint32_t row_bytes = (uint32_t)(K * ES);
-    const int kb = K >> 5;
+    const int kb = K >> 5, kt128 = K >> 7;
     setup_ring_loader<DT, RB>(
         ld, lay, tid, row_bytes, ntf0, ntf1,
         [&](int row) { return (uint32_t)max(ri.tok[row], 0) * row_bytes; },  // dead rows read token 0
-        a.x_scales, [&](int row) { return (uint32_t)max(ri.tok[row], 0) * (uint32_t)kb; },
+        reinterpret_cast<const uint8_t *>(a.xs_tiled + (int64_t)first * kt128 * kBlockRows),
+        [&](int row) { return (uint32_t)(((row >> 7) * kt128 * kBlockRows + (row & 127)) * 4); },
         a.w1_scales + (int64_t)e * N * kb,
         [&](int row) { return (uint32_t)blocked_scale_off((row < 128 ? h0 : H + h0 - 128) + row, 0, K >> 7); });
 
@@ -475,10 +481,11 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     ld.w_base[0] = a.w2 + ((int64_t)e * K + k0) * H * ES;
     ld.w_base[1] = (k0 + 128 < K) ? ld.w_base[0] + (int64_t)128 * H * ES : ld.w_base[0];
     const uint32_t row_bytes = (uint32_t)(H * ES);
-    const int hb = H >> 5;
+    const int hb = H >> 5, ht128 = H >> 7;
     setup_ring_loader<DT, RB>(
         ld, lay, tid, row_bytes, ntf0, ntf1, [&](int row) { return (uint32_t)row * row_bytes; },
-        a.act_scales + row0 * hb, [&](int row) { return (uint32_t)row * (uint32_t)hb; },
+        reinterpret_cast<const uint8_t *>(a.act_scales + (int64_t)first * ht128 * kBlockRows),
+        [&](int row) { return (uint32_t)(((row >> 7) * ht128 * kBlockRows + (row & 127)) * 4); },
         a.w2_scales + (int64_t)e * K * hb,
         [&](int row) { return (uint32_t)blocked_scale_off(min(k0 + row, K - 1), 0, H >> 7); });
 
@@ -595,7 +602,8 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
                                                            int2 *work_up, int n_wt_up, int grid_up, int2 *work_down,
                                                            int n_wt_down, int grid_down, int num_experts,
                                                            const int32_t *sorted_ids, int sorted_num, int32_t *inv,
-                                                           int n_pairs, int do_invert) {
+                                                           int n_pairs, int do_invert, const uint8_t *x_scales,
+                                                           uint32_t *xs_tiled, int nkt, int top_k, int M) {
     if (blockIdx.x == 0 && tiles != nullptr) {
         __shared__ int s_max[4], s_sum[4], s_carry[2];
         const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -657,6 +665,43 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
             if (p >= 0 && p < n_pairs) inv[p] = s;
         }
     }
+    if (do_invert && xs_tiled != nullptr) {
+        // mxfp8: the e8m0 scales of the gathered x rows, re-tiled for the up kernel's loader (see
+        // MoeArgs::xs_tiled); rows without a token get 2^0.  One sorted block per turn, through LDS so
+        // that both the reads (a row's scales) and the writes (128 rows of one K tile) are contiguous.
+        // Workgroup 0 builds the tiles above and takes no share unless it is alone.
+        __shared__ int s_tok[kBlockRows];
+        __shared__ uint32_t s_sc[kBlockRows][65];
+        const int tid = threadIdx.x;
+        const int n_live = min((ntpp[0] + kBlockRows - 1) / kBlockRows, n_blocks);
+        const int workers = gridDim.x > 1 ? (int)gridDim.x - 1 : 1;
+        const int me = gridDim.x > 1 ? (int)blockIdx.x - 1 : 0;
+        const uint32_t *xs = reinterpret_cast<const uint32_t *>(x_scales);  // nkt dwords per token
+        for (int b = me; b >= 0 && b < n_live; b += workers) {
+            if (tid < kBlockRows) {
+                const int srow = b * kBlockRows + tid;
+                const int p = srow < sorted_num ? sorted_ids[srow] : -1;
+                int tok = p >= 0 ? p / top_k : -1;
+                if (tok >= M) tok = -1;
+                s_tok[tid] = tok;
+            }
+            __syncthreads();
+            for (int c0 = 0; c0 < nkt; c0 += 64) {
+                const int cw = min(64, nkt - c0);
+                for (int i = tid; i < kBlockRows * cw; i += 256) {
+                    const int r = i / cw, c = i - r * cw;
+                    const int tok = s_tok[r];
+                    s_sc[r][c] = tok >= 0 ? xs[(int64_t)tok * nkt + c0 + c] : 0x7f7f7f7fu;
+                }
+                __syncthreads();
+                for (int i = tid; i < kBlockRows * cw; i += 256) {
+                    const int c = i >> 7, r = i & 127;
+                    xs_tiled[((int64_t)b * nkt + c0 + c) * kBlockRows + r] = s_sc[r][c];
+                }
+                __syncthreads();
+            }
+        }
+    }
 }
 
 // out[t, 8 columns] = bf16(sum over the token's top_k pairs p, in pair order, of w[p] * y[row(p)])
@@ -705,7 +750,7 @@ __global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int3
 // ------------------------------------------------------------------------------------------ host
 
 struct WorkspaceLayout {
-    size_t n_tiles_off, tiles_off, work_up_off, work_down_off, inv_off, y_off, act_off, act_scales_off, total;
+    size_t n_tiles_off, tiles_off, work_up_off, work_down_off, inv_off, y_off, act_off, act_scales_off, xs_tiled_off, total;
 };
 
 static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_num, int top_k) {
@@ -730,6 +775,8 @@ static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_
     off = align_up(off + rows * H * (dt == DT_BF16 ? 2 : 1), 256);
     l.act_scales_off = off;
     if (dt == DT_FP8) off = align_up(off + rows * (H / 32), 256);
+    l.xs_tiled_off = off;
+    if (dt == DT_FP8) off = align_up(off + rows * ((size_t)K / 32), 256);
     l.total = off;
     return l;
 }
@@ -763,7 +810,8 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
         hipLaunchKernelGGL(moe_prologue_kernel, dim3(blocks), dim3(256), 0, s, a.expert_ids, a.ntpp, a.n_blocks,
                            sb.tiles, sb.n_tiles, sb.work_up, a.n_wtiles, grid_for(a.n_blocks * a.n_wtiles),
                            sb.work_down, n_wt_down, grid_for(a.n_blocks * n_wt_down), a.E,
-                           a.sorted_ids, a.sorted_num, a.inv, a.M * a.top_k, do_invert);
+                           a.sorted_ids, a.sorted_num, a.inv, a.M * a.top_k, do_invert, a.x_scales, a.xs_tiled,
+                           a.K >> 7, a.top_k, a.M);
     }
     if (a.n_blocks > 0) {
         a.work = sb.work_up;
@@ -895,7 +943,8 @@ extern "C" int pmoe_fused_moe_mxfp8(const void *x, const void *x_scales, const v
     a.y = ws + l.y_off;
     a.inv = reinterpret_cast<int32_t *>(ws + l.inv_off);
     a.act = ws + l.act_off;
-    a.act_scales = reinterpret_cast<uint8_t *>(ws + l.act_scales_off);
+    a.act_scales = reinterpret_cast<uint32_t *>(ws + l.act_scales_off);
+    a.xs_tiled = reinterpret_cast<uint32_t *>(ws + l.xs_tiled_off);
     a.top_k = top_k; a.M = M; a.K = K; a.N = N; a.H = N / 2; a.E = num_experts; a.sorted_num = sorted_num;
     return launch_pipeline<DT_FP8>(a, sched_buffers(ws, l), out, split, static_cast<hipStream_t>(stream));
 }

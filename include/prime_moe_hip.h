@@ -125,6 +125,13 @@ int pmoe_quantize_mx(const void *src_bf16, void *q, void *scales, int64_t rows, 
 void pmoe_set_phase_mask(int mask);
 
 /*
+ * Tuning and test aid with no counterpart in the reference: the number of consecutive weight tiles
+ * (1..16) one workgroup of the mxfp8 up and down kernels takes for its row tile, for the calling
+ * thread; 0 (the default) lets every launch choose from its sizes.  The result does not depend on it.
+ */
+void pmoe_set_tiles_per_workgroup(int n);
+
+/*
  * Second profiling aid without a counterpart in the reference: a plain device copy of `bytes`
  * bytes (multiple of 16) done by a kernel named copy_calibration_kernel.  Its known traffic
  * (bytes read, bytes written) scales the FETCH_SIZE / WRITE_SIZE hardware counters of a

@@ -63,15 +63,17 @@ constexpr int kPartRB = PMOE_PART_RB;      // of mxfp8 tiles with more, short of
 constexpr int kActPitchBf16 = 272;  // 128 bf16 + 16 B pad: 16-byte aligned rows, 2-way conflicts at most
 constexpr int kActPitchFp8 = 144;   // 128 e4m3 + 16 B pad
 
-// Workgroup id -> (first block, blocks, weight tile, expert): one load from the work list, which the
-// prologue lays out by workgroup id (see emit_work); entries of workgroups without a tile are -1.
-__device__ __forceinline__ bool resolve_tile(const MoeArgs &a, int &first, int &nb, int &wt, int &e) {
+// Workgroup id -> (first block, blocks, first weight tile, expert, number of weight tiles): one load
+// from the work list, which the prologue lays out by workgroup id (see emit_work); entries of
+// workgroups without work are -1.
+__device__ __forceinline__ bool resolve_tile(const MoeArgs &a, int &first, int &nb, int &wt, int &e, int &n_sub) {
     const int2 w = a.work[blockIdx.x];
     if (w.x < 0) return false;
     first = w.x & 0x0fffffff;
     nb = w.x >> 28;
     wt = w.y & 0xffff;
-    e = w.y >> 16;
+    e = (w.y >> 16) & 0x3ff;
+    n_sub = ((w.y >> 26) & 0xf) + 1;
     return true;
 }
 
@@ -267,9 +269,10 @@ __device__ __forceinline__ void store_act_tile(const MoeArgs &a, const char *til
 // K tile lies 512 bytes on in both (blocked weight scales, tiled token-side scales).  Only the live 32-row
 // fragments of the two blocks (ntf0, ntf1 of them) are copied; they are packed one after the other in
 // the stage (see ring::Layout).
-template <int DT, int RB, typename TokOff, typename TokScOff, typename WScOff>
+template <int DT, int RB, bool FULL, typename TokOff, typename TokScOff, typename WScOff>
 __device__ __forceinline__ void setup_ring_loader(ring::Loader<RB> &ld, const ring::Layout &lay, int tid,
-                                                  uint32_t w_pitch, int ntf0, int ntf1, TokOff tok_row_off,
+                                                  uint32_t w_pitch, int ntf0, int ntf1, const RowInfo<2> &ri,
+                                                  TokOff tok_row_off,
                                                   const uint8_t *tok_sc_base, TokScOff tok_sc_off,
                                                   const uint8_t *w_sc_base, WScOff w_sc_off) {
     using L = ring::Loader<RB>;
@@ -285,11 +288,14 @@ __device__ __forceinline__ void setup_ring_loader(ring::Loader<RB> &ld, const ri
         const int frag = row0 >> 5;  // the instruction's rows lie in this 32-row fragment
         ld.tok_dst[0][q] = ld.tok_dst[1][q] = -1;
         ld.tok_off[0][q] = ld.tok_off[1][q] = 0;
-        if (frag < ntf0) {
+        // (the constant wait counts of full tiles assume every instruction: those copy all their rows)
+        ld.tok_live[0][q] = frag < ntf0 && (FULL || ri.tok[row] >= 0);
+        ld.tok_live[1][q] = frag < ntf1 && (FULL || ri.tok[kBlockRows + row] >= 0);
+        if (__ballot(ld.tok_live[0][q]) != 0) {
             ld.tok_dst[0][q] = row0 * RB;
             ld.tok_off[0][q] = tok_row_off(row) + gchunk;
         }
-        if (frag < ntf1) {
+        if (__ballot(ld.tok_live[1][q]) != 0) {
             ld.tok_dst[1][q] = lay.group1_off + row0 * RB;
             ld.tok_off[1][q] = tok_row_off(kBlockRows + row) + gchunk;
         }
@@ -338,49 +344,71 @@ __device__ __forceinline__ int slab_rotation(int n_slabs) {
 // wave v of a group owns gate/up rows 32v..32v+31 so gate and up of one activation element sit in the
 // same lane and register.
 template <int DT, int RB, int NTF, bool FULL>
-__device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht, int e, RowInfo<2> &ri,
+__device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht, int n_sub, int e, RowInfo<2> &ri,
                                              char *lds, uint32_t *act_sc_lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
     const int K = a.K, H = a.H, N = a.N;
-    const int h0 = ht * 128;
     const int ntf0 = __builtin_amdgcn_readfirstlane((ri.nvalid[0] + 31) >> 5);
     const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
     const int my_ntf = grp ? ntf1 : ntf0;
     const bool active = my_ntf > 0;
     const ring::Layout lay = ring::make_layout<DT, RB>(ntf0, ntf1, ring::ring_bytes<DT>());
 
+    int h0 = ht * 128;
     ring::Loader<RB> ld;
     ld.tok_base = a.x;
     ld.w_base[0] = a.w1 + ((int64_t)e * N + h0) * K * ES;
     ld.w_base[1] = ld.w_base[0] + (int64_t)H * K * ES;
     const uint32_t row_bytes = (uint32_t)(K * ES);
     const int kb = K >> 5, kt128 = K >> 7;
-    setup_ring_loader<DT, RB>(
-        ld, lay, tid, row_bytes, ntf0, ntf1,
-        [&](int row) { return (uint32_t)max(ri.tok[row], 0) * row_bytes; },  // dead rows read token 0
+    setup_ring_loader<DT, RB, FULL>(
+        ld, lay, tid, row_bytes, ntf0, ntf1, ri,
+        [&](int row) { return (uint32_t)max(ri.tok[row], 0) * row_bytes; },
         reinterpret_cast<const uint8_t *>(a.xs_tiled + (int64_t)first * kt128 * kBlockRows),
         [&](int row) { return (uint32_t)(((row >> 7) * kt128 * kBlockRows + (row & 127)) * 4); },
         a.w1_scales + (int64_t)e * N * kb,
         [&](int row) { return (uint32_t)blocked_scale_off((row < 128 ? h0 : H + h0 - 128) + row, 0, K >> 7); });
 
     const int wrow[2] = {32 * w4, 128 + 32 * w4};
-    f32x16 acc[2][4];
-    zero_acc(acc);
     const int n_slabs = (K * ES) / RB;
     const int start = slab_rotation<RB>(n_slabs);
     const int tok_region = grp ? lay.group1_off : 0;
-    if (active) ring::main_loop<DT, RB, NTF, true, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
-    else ring::main_loop<DT, RB, NTF, true, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
-
-    // the ring is free (main_loop ends with a barrier): reuse it for the activation tiles
+    // the ring is free after main_loop (it ends with a barrier): its head holds the activation tiles
     constexpr int kPitch = DT == DT_BF16 ? kActPitchBf16 : kActPitchFp8;
     char *tile = lds + grp * (kBlockRows * kPitch);
     uint32_t *sc_tile = act_sc_lds + grp * kBlockRows;
-    if (active) swiglu_epilogue<DT, NTF>(acc, tile, sc_tile, w4, lane);
-    __syncthreads();
-    if (active) store_act_tile<DT>(a, tile, sc_tile, (int64_t)(first + grp) * kBlockRows, h0, my_ntf, gt);
+    const int SB = ring::stage_bytes<DT, RB, FULL>(lay), NS = ring::stage_count<DT, RB, FULL>(lay);
+    // first stage clear of the activation tiles: the next weight tile's copies start there, under
+    // the epilogue of this one
+    const int epi_bytes = (ntf1 > 0 ? 2 : 1) * kBlockRows * kPitch;
+    const int free0 = (epi_bytes + SB - 1) / SB;
+    int stage0 = 0, n_pre = 0;
+    for (int sub = 0; sub < n_sub; ++sub) {
+        f32x16 acc[2][4];
+        zero_acc(acc);
+        if (active)
+            ring::main_loop<DT, RB, NTF, true, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
+        else
+            ring::main_loop<DT, RB, NTF, true, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
+        const bool more = sub + 1 < n_sub;
+        if (more) {
+            // same token rows, the next 128 gate and 128 up rows of the expert
+            ld.w_base[0] += (int64_t)128 * K * ES;
+            ld.w_base[1] += (int64_t)128 * K * ES;
+            if (DT == DT_FP8 && wave >= 4) ld.sc_off += (uint32_t)kt128 * 512u;
+            ld.make_uniform();
+            stage0 = free0 < NS ? free0 : 0;
+            n_pre = free0 < NS ? min(NS - 1, NS - free0) : 0;
+            ring::pre_issue<DT, RB, FULL>(ld, lay, lds, n_slabs, start, stage0, n_pre);
+        }
+        if (active) swiglu_epilogue<DT, NTF>(acc, tile, sc_tile, w4, lane);
+        __syncthreads();
+        if (active) store_act_tile<DT>(a, tile, sc_tile, (int64_t)(first + grp) * kBlockRows, h0, my_ntf, gt);
+        if (more) __syncthreads();  // the tiles have been read: the head of the ring may be filled again
+        h0 += 128;
+    }
 }
 
 // LDS plan of the split kernels.  bf16: the 160 KB ring of the wide engine is all the LDS there is;
@@ -439,35 +467,35 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
     using L = SplitLds<DT>;
     __shared__ __attribute__((aligned(1024))) char lds[L::kTotal];
     RowInfo<2> &ri = *reinterpret_cast<RowInfo<2> *>(lds + L::kRowInfoOff);
-    int first, nb, ht, e;
-    if (!resolve_tile(a, first, nb, ht, e)) return;
+    int first, nb, ht, e, n_sub;
+    if (!resolve_tile(a, first, nb, ht, e, n_sub)) return;
     const int ntf = load_row_info<2>(a, first, nb, ri);
     if (ntf == 0) return;
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
-    if constexpr (DT == DT_BF16) {
-        if (skinny) up_tile_ring<DT, kSkinnyRB, 1, false>(a, first, ht, e, ri, lds, nullptr);
+    if constexpr (DT == DT_BF16) {  // one weight tile per workgroup on this path (see launch_pipeline)
+        if (skinny) up_tile_ring<DT, kSkinnyRB, 1, false>(a, first, ht, 1, e, ri, lds, nullptr);
         else if (ntf == 1) up_tile_wide_bf16<1>(a, first, ht, e, ri, lds);
         else if (ntf == 2) up_tile_wide_bf16<2>(a, first, ht, e, ri, lds);
         else up_tile_wide_bf16<4>(a, first, ht, e, ri, lds);
     } else {
         uint32_t *act_sc_lds = reinterpret_cast<uint32_t *>(lds + L::kActScaleOff);
         const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-        if (ntf == 1) up_tile_ring<DT, kSkinnyRB, 1, false>(a, first, ht, e, ri, lds, act_sc_lds);
-        else if (ntf == 2) up_tile_ring<DT, kPartRB, 2, false>(a, first, ht, e, ri, lds, act_sc_lds);
-        else if (full) up_tile_ring<DT, 64, 4, true>(a, first, ht, e, ri, lds, act_sc_lds);
-        else up_tile_ring<DT, kPartRB, 4, false>(a, first, ht, e, ri, lds, act_sc_lds);
+        if (ntf == 1) up_tile_ring<DT, kSkinnyRB, 1, false>(a, first, ht, n_sub, e, ri, lds, act_sc_lds);
+        else if (ntf == 2) up_tile_ring<DT, kPartRB, 2, false>(a, first, ht, n_sub, e, ri, lds, act_sc_lds);
+        else if (full) up_tile_ring<DT, 64, 4, true>(a, first, ht, n_sub, e, ri, lds, act_sc_lds);
+        else up_tile_ring<DT, kPartRB, 4, false>(a, first, ht, n_sub, e, ri, lds, act_sc_lds);
     }
 }
 
 // Down kernel of the split pipeline: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
 // full reduction over H inside the workgroup (no split-K), then w[row] * y added to accum[token].
 template <int DT, int RB, int NTF, bool FULL>
-__device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, char *lds) {
+__device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int kt, int n_sub, int e, RowInfo<2> &ri,
+                                               char *lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
     const int K = a.K, H = a.H;
-    const int k0 = kt * kWRows;
     const int64_t row0 = (int64_t)first * kBlockRows;
     const int ntf0 = __builtin_amdgcn_readfirstlane((ri.nvalid[0] + 31) >> 5);
     const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
@@ -476,35 +504,63 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     const bool active = my_ntf > 0;
     const ring::Layout lay = ring::make_layout<DT, RB>(ntf0, ntf1, ring::ring_bytes<DT>());
 
-    ring::Loader<RB> ld;
-    ld.tok_base = a.act + row0 * H * ES;
-    ld.w_base[0] = a.w2 + ((int64_t)e * K + k0) * H * ES;
-    ld.w_base[1] = (k0 + 128 < K) ? ld.w_base[0] + (int64_t)128 * H * ES : ld.w_base[0];
+    int k0 = kt * kWRows;
     const uint32_t row_bytes = (uint32_t)(H * ES);
     const int hb = H >> 5, ht128 = H >> 7;
-    setup_ring_loader<DT, RB>(
-        ld, lay, tid, row_bytes, ntf0, ntf1, [&](int row) { return (uint32_t)row * row_bytes; },
+    ring::Loader<RB> ld;
+    ld.tok_base = a.act + row0 * H * ES;
+    // weight rows (output columns) k0 .. k0 + 255 of the expert; the last tile of a K that is not a
+    // multiple of 256 has 128 of them and reads the first half twice
+    auto set_weights = [&](int k) {
+        ld.w_base[0] = a.w2 + ((int64_t)e * K + k) * H * ES;
+        ld.w_base[1] = (k + 128 < K) ? ld.w_base[0] + (int64_t)128 * H * ES : ld.w_base[0];
+        if (DT == DT_FP8 && wave >= 4)
+            ld.sc_off = (uint32_t)blocked_scale_off(min(k + 64 * (wave - 4) + lane, K - 1), 0, ht128);
+    };
+    set_weights(k0);
+    setup_ring_loader<DT, RB, FULL>(
+        ld, lay, tid, row_bytes, ntf0, ntf1, ri, [&](int row) { return (uint32_t)row * row_bytes; },
         reinterpret_cast<const uint8_t *>(a.act_scales + (int64_t)first * ht128 * kBlockRows),
         [&](int row) { return (uint32_t)(((row >> 7) * ht128 * kBlockRows + (row & 127)) * 4); },
         a.w2_scales + (int64_t)e * K * hb,
-        [&](int row) { return (uint32_t)blocked_scale_off(min(k0 + row, K - 1), 0, H >> 7); });
+        [&](int row) { return (uint32_t)blocked_scale_off(min(k0 + row, K - 1), 0, ht128); });
 
     const int wrow[2] = {64 * w4, 64 * w4 + 32};
-    f32x16 acc[2][4];
-    zero_acc(acc);
     const int n_slabs = (H * ES) / RB;
     const int start = slab_rotation<RB>(n_slabs);
     const int tok_region = grp ? lay.group1_off : 0;
-    if (active) ring::main_loop<DT, RB, NTF, true, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
-    else ring::main_loop<DT, RB, NTF, true, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start);
-    // the ring is free (main_loop ends with a barrier): reuse it for the two 128 x 256 output tiles
-    if constexpr (NTF == 1) {
-        if (active) store_y_direct(a, acc, row0 + grp * kBlockRows, k0, my_rows, w4, lane);
-    } else {
-        char *tile = lds + grp * (kBlockRows * kYPitch);
-        if (active) y_epilogue<NTF>(acc, tile, w4, lane);
-        __syncthreads();
-        if (active) store_y_tile(a, tile, row0 + grp * kBlockRows, k0, my_rows, gt);
+    const int SB = ring::stage_bytes<DT, RB, FULL>(lay), NS = ring::stage_count<DT, RB, FULL>(lay);
+    // the ring is free after main_loop (it ends with a barrier): its head holds the 128 x 256 output
+    // tiles of the live groups (none for tiles of one fragment, which store from registers); the
+    // next weight tile's copies start in the first stage clear of them, under this tile's epilogue
+    const int epi_bytes = NTF == 1 ? 0 : (ntf1 > 0 ? 2 : 1) * kBlockRows * kYPitch;
+    const int free0 = (epi_bytes + SB - 1) / SB;
+    int stage0 = 0, n_pre = 0;
+    for (int sub = 0; sub < n_sub; ++sub) {
+        f32x16 acc[2][4];
+        zero_acc(acc);
+        if (active)
+            ring::main_loop<DT, RB, NTF, true, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
+        else
+            ring::main_loop<DT, RB, NTF, true, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
+        const bool more = sub + 1 < n_sub;
+        if (more) {
+            set_weights(k0 + kWRows);
+            ld.make_uniform();
+            stage0 = free0 < NS ? free0 : 0;
+            n_pre = free0 < NS ? min(NS - 1, NS - free0) : 0;
+            ring::pre_issue<DT, RB, FULL>(ld, lay, lds, n_slabs, start, stage0, n_pre);
+        }
+        if constexpr (NTF == 1) {
+            if (active) store_y_direct(a, acc, row0 + grp * kBlockRows, k0, my_rows, w4, lane);
+        } else {
+            char *tile = lds + grp * (kBlockRows * kYPitch);
+            if (active) y_epilogue<NTF>(acc, tile, w4, lane);
+            __syncthreads();
+            if (active) store_y_tile(a, tile, row0 + grp * kBlockRows, k0, my_rows, gt);
+            if (more) __syncthreads();  // the tiles have been read: the head of the ring may be filled again
+        }
+        k0 += kWRows;
     }
 }
 
@@ -552,22 +608,22 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
     using L = SplitLds<DT>;
     __shared__ __attribute__((aligned(1024))) char lds[L::kTotal];
     RowInfo<2> &ri = *reinterpret_cast<RowInfo<2> *>(lds + L::kRowInfoOff);
-    int first, nb, kt, e;
-    if (!resolve_tile(a, first, nb, kt, e)) return;
+    int first, nb, kt, e, n_sub;
+    if (!resolve_tile(a, first, nb, kt, e, n_sub)) return;
     const int ntf = load_row_info<2>(a, first, nb, ri);
     if (ntf == 0) return;
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
-    if constexpr (DT == DT_BF16) {
-        if (skinny) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, e, ri, lds);
+    if constexpr (DT == DT_BF16) {  // one weight tile per workgroup on this path (see launch_pipeline)
+        if (skinny) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, 1, e, ri, lds);
         else if (ntf == 1) down_tile_wide_bf16<1>(a, first, kt, e, ri, lds);
         else if (ntf == 2) down_tile_wide_bf16<2>(a, first, kt, e, ri, lds);
         else down_tile_wide_bf16<4>(a, first, kt, e, ri, lds);
     } else {
         const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-        if (ntf == 1) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, e, ri, lds);
-        else if (ntf == 2) down_tile_ring<DT, kPartRB, 2, false>(a, first, kt, e, ri, lds);
-        else if (full) down_tile_ring<DT, 64, 4, true>(a, first, kt, e, ri, lds);
-        else down_tile_ring<DT, kPartRB, 4, false>(a, first, kt, e, ri, lds);
+        if (ntf == 1) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, n_sub, e, ri, lds);
+        else if (ntf == 2) down_tile_ring<DT, kPartRB, 2, false>(a, first, kt, n_sub, e, ri, lds);
+        else if (full) down_tile_ring<DT, 64, 4, true>(a, first, kt, n_sub, e, ri, lds);
+        else down_tile_ring<DT, kPartRB, 4, false>(a, first, kt, n_sub, e, ri, lds);
     }
 }
 
@@ -580,15 +636,18 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
 // Hardware hands consecutive workgroup ids to the 8 XCDs round-robin, so position `l` of the walk
 // is given to workgroup id 8 * (l mod per_xcd) + l / per_xcd: one XCD then runs a contiguous range of
 // the walk.  The entry carries everything the workgroup needs to start: (first block | blocks << 28,
-// weight tile | expert << 16).
-__device__ __forceinline__ void emit_work(int2 *work, int n_wt, int tile, int n_tiles, int first, int nb, int e) {
+// first weight tile | expert << 16 | (weight tiles - 1) << 26); experts < 1024, up to 16 weight tiles.
+__device__ __forceinline__ void emit_work(int2 *work, int n_wt, int per_job, int tile, int n_tiles, int first, int nb,
+                                          int e) {
     constexpr int GW = 8;
-    const int per_xcd = (n_tiles * n_wt + 7) >> 3;
-    for (int wt = 0; wt < n_wt; ++wt) {
-        const int wg = wt / GW;
-        const int gw = min(GW, n_wt - wg * GW);
-        const int l = wg * GW * n_tiles + tile * gw + (wt - wg * GW);
-        work[8 * (l % per_xcd) + l / per_xcd] = make_int2(first | (nb << 28), wt | (e << 16));
+    const int n_jobs = (n_wt + per_job - 1) / per_job;  // a workgroup takes `per_job` consecutive weight tiles
+    const int per_xcd = (n_tiles * n_jobs + 7) >> 3;
+    for (int j = 0; j < n_jobs; ++j) {
+        const int wg = j / GW;
+        const int gw = min(GW, n_jobs - wg * GW);
+        const int l = wg * GW * n_tiles + tile * gw + (j - wg * GW);
+        const int wt = j * per_job, cnt = min(per_job, n_wt - wt);
+        work[8 * (l % per_xcd) + l / per_xcd] = make_int2(first | (nb << 28), wt | (e << 16) | ((cnt - 1) << 26));
     }
 }
 
@@ -599,8 +658,9 @@ __device__ __forceinline__ void emit_work(int2 *work, int n_wt, int tile, int n_
 // in the schedule keep whatever the buffer held; the reader validates an entry against sorted_ids.
 __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert_ids, const int32_t *ntpp,
                                                            int n_blocks, int2 *tiles, int *n_tiles,
-                                                           int2 *work_up, int n_wt_up, int grid_up, int2 *work_down,
-                                                           int n_wt_down, int grid_down, int num_experts,
+                                                           int2 *work_up, int n_wt_up, int per_job_up, int grid_up,
+                                                           int2 *work_down, int n_wt_down, int per_job_down,
+                                                           int grid_down, int num_experts,
                                                            const int32_t *sorted_ids, int sorted_num, int32_t *inv,
                                                            int n_pairs, int do_invert, const uint8_t *x_scales,
                                                            uint32_t *xs_tiled, int nkt, int top_k, int M) {
@@ -653,8 +713,8 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
             const int2 tl = tiles[t];
             const int e = expert_ids[tl.x];
             if (e < 0 || e >= num_experts) continue;  // nothing to compute for a block without an expert
-            emit_work(work_up, n_wt_up, t, nt, tl.x, tl.y, e);
-            emit_work(work_down, n_wt_down, t, nt, tl.x, tl.y, e);
+            emit_work(work_up, n_wt_up, per_job_up, t, nt, tl.x, tl.y, e);
+            emit_work(work_down, n_wt_down, per_job_down, t, nt, tl.x, tl.y, e);
         }
     }
     if (do_invert) {
@@ -783,9 +843,39 @@ static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_
 
 static int grid_for(int n_tiles) { return (n_tiles + 7) / 8 * 8; }
 
+// CU count of the current device, rounded down to a multiple of the 8 XCDs.
+static int resident_grid() {
+    static thread_local int cached_dev = -1, cached = 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (dev != cached_dev) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 8) cus = 256;
+        cached = cus / 8 * 8;
+        cached_dev = dev;
+    }
+    return cached;
+}
+
 // Which phases of the pipeline the fused entry points enqueue (all by default); see
 // pmoe_set_phase_mask in the header.
 static thread_local int g_phase_mask = PMOE_PHASE_ALL;
+// Weight tiles a workgroup of the mxfp8 kernels takes in a row (0: chosen per launch); see
+// pmoe_set_tiles_per_workgroup in the header.
+static thread_local int g_tiles_per_wg = 0;
+
+// A workgroup of the mxfp8 kernels can keep its token rows and take several weight tiles in a row: it
+// saves the set-up of all but the first and starts each tile's copies under the epilogue of the one
+// before, but the coarser work balances worse over the CUs.  Measured on the DeepSeek-V3-like prefill
+// and decode shapes: two tiles gain 3 % on the down kernel (16 slabs per tile), nothing on the up kernel
+// (56 slabs per tile), more than two lose on both.  So: two for the down kernel when that still leaves
+// 8 rounds of workgroups per CU, one otherwise.  The bf16 kernels take one (their wide tiles run on the
+// unit ring, which has no such hand-over).
+static int tiles_per_workgroup(int dt, bool down, int n_blocks, int n_wt) {
+    if (dt != DT_FP8) return 1;
+    if (g_tiles_per_wg > 0) return std::min(g_tiles_per_wg, n_wt);
+    return (down && (int64_t)n_blocks * n_wt >= (int64_t)resident_grid() * 16) ? 2 : 1;
+}
 
 struct SchedBuffers {
     int2 *tiles;
@@ -803,25 +893,29 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
     a.tiles = sb.tiles;
     a.n_tiles = sb.n_tiles;
     const int n_wt_down = (a.K + kWRows - 1) / kWRows;
+    const int per_up = tiles_per_workgroup(DT, false, a.n_blocks, a.n_wtiles);
+    const int per_down = tiles_per_workgroup(DT, true, a.n_blocks, n_wt_down);
+    const int grid_up = grid_for(a.n_blocks * ((a.n_wtiles + per_up - 1) / per_up));
+    const int grid_down = grid_for(a.n_blocks * ((n_wt_down + per_down - 1) / per_down));
     {
         // the work lists are needed by the two kernels even when the rest of the prologue is masked off
         const int do_invert = (mask & PMOE_PHASE_PROLOGUE) ? 1 : 0;
         const int blocks = do_invert ? std::max(1, std::min((a.sorted_num + 255) / 256, 1024)) : 1;
         hipLaunchKernelGGL(moe_prologue_kernel, dim3(blocks), dim3(256), 0, s, a.expert_ids, a.ntpp, a.n_blocks,
-                           sb.tiles, sb.n_tiles, sb.work_up, a.n_wtiles, grid_for(a.n_blocks * a.n_wtiles),
-                           sb.work_down, n_wt_down, grid_for(a.n_blocks * n_wt_down), a.E,
+                           sb.tiles, sb.n_tiles, sb.work_up, a.n_wtiles, per_up, grid_up,
+                           sb.work_down, n_wt_down, per_down, grid_down, a.E,
                            a.sorted_ids, a.sorted_num, a.inv, a.M * a.top_k, do_invert, a.x_scales, a.xs_tiled,
                            a.K >> 7, a.top_k, a.M);
     }
     if (a.n_blocks > 0) {
         a.work = sb.work_up;
         if (mask & PMOE_PHASE_UP)
-            hipLaunchKernelGGL((moe_up_kernel<DT>), dim3(grid_for(a.n_blocks * a.n_wtiles)), dim3(512), 0, s, a);
+            hipLaunchKernelGGL((moe_up_kernel<DT>), dim3(grid_up), dim3(512), 0, s, a);
         MoeArgs d = a;
         d.n_wtiles = n_wt_down;
         d.work = sb.work_down;
         if (mask & PMOE_PHASE_DOWN)
-            hipLaunchKernelGGL((moe_down_kernel<DT>), dim3(grid_for(d.n_blocks * d.n_wtiles)), dim3(512), 0, s, d);
+            hipLaunchKernelGGL((moe_down_kernel<DT>), dim3(grid_down), dim3(512), 0, s, d);
     }
     if (mask & PMOE_PHASE_FINALIZE) {
         const int64_t n8 = n_out / 8;
@@ -850,6 +944,7 @@ static SchedBuffers sched_buffers(char *ws, const WorkspaceLayout &l) {
 using namespace pmoe;
 
 extern "C" void pmoe_set_phase_mask(int mask) { g_phase_mask = mask; }
+extern "C" void pmoe_set_tiles_per_workgroup(int n) { g_tiles_per_wg = n < 0 ? 0 : (n > 16 ? 16 : n); }
 
 extern "C" size_t pmoe_fused_moe_bf16_workspace_bytes(int M, int K, int N, int num_experts,
                                                       int sorted_num, int top_k, int split) {
@@ -887,6 +982,7 @@ extern "C" int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2,
     PMOE_REQUIRE(bpc == 1 && cpc == 1, "bpc=cpc=1 is the only supported configuration");
     PMOE_REQUIRE(!split || stages <= 4, "split=True requires stages<=4, got stages=%d", stages);
     PMOE_REQUIRE(top_k > 0 && num_experts > 0 && sorted_num >= 0, "fused_moe_bf16: bad top_k / num_experts / sorted_num");
+    PMOE_REQUIRE(num_experts <= 1024, "fused_moe_bf16: at most 1024 experts, got %d", num_experts);
     PMOE_REQUIRE(x && w && w2 && out && sorted_token_ids && expert_idxs && num_tokens_post_padded && topk_weights,
                  "fused_moe_bf16: null pointer");
     const WorkspaceLayout l = workspace_layout(DT_BF16, M, K, N, sorted_num, top_k);
@@ -922,6 +1018,7 @@ extern "C" int pmoe_fused_moe_mxfp8(const void *x, const void *x_scales, const v
     if (int rc = check_tuning("fused_moe_mxfp8", block_m, block_n, warp_n, stages, 4)) return rc;
     PMOE_REQUIRE(bpc == 1, "mxfp8 supports bpc=1 only");
     PMOE_REQUIRE(top_k > 0 && num_experts > 0 && sorted_num >= 0, "fused_moe_mxfp8: bad top_k / num_experts / sorted_num");
+    PMOE_REQUIRE(num_experts <= 1024, "fused_moe_mxfp8: at most 1024 experts, got %d", num_experts);
     PMOE_REQUIRE(x && x_scales && w && w_scales && w2 && w2_scales && out && sorted_token_ids && expert_idxs &&
                      num_tokens_post_padded && topk_weights,
                  "fused_moe_mxfp8: null pointer");

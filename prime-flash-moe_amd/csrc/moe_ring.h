@@ -119,7 +119,9 @@ __device__ __forceinline__ void wait_and_barrier_dyn(int n) {
 // Per-thread description of the copies of one stage.  A 128-row block of token rows or half of the
 // weight tile takes N = RB / 64 instructions of every wave: instruction q of wave w moves rows
 // q * 8 * rpc + rpc * w .. + rpc - 1 of it (rpc = 1024 / RB rows per instruction).  Token rows of
-// fragments without live rows are not copied.  Scales: at most one 4-byte-per-lane instruction per
+// fragments without live rows are not copied, nor are the rows without a token inside a live fragment
+// (an instruction whose rows all lack one is dropped: the wait counts rely on every issued
+// instruction having an active lane).  Scales: at most one 4-byte-per-lane instruction per
 // wave.
 template <int RB>
 struct Loader {
@@ -133,6 +135,8 @@ struct Loader {
     uint32_t sc_off;      // this lane's row in them
     uint32_t sc_step;     // bytes between consecutive 128-wide K tiles: 4 (row major) or 512 (blocked)
     int tok_dst[2][N];    // LDS offset inside a stage of this wave's token rows; -1: nothing to copy
+    bool tok_live[2][N];  // this lane's row holds a token (rows without one are not fetched: what the
+                          // stage holds for them only reaches their own, unused, output rows)
     int w_dst[2][N];      // LDS offsets of this wave's weight rows
     int sc_dst;           // LDS offset of this wave's scale dwords; -1: none
     int lps;              // copy instructions this wave issues per stage
@@ -154,7 +158,9 @@ struct Loader {
         for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int q = 0; q < N; ++q)
-                if (tok_dst[b][q] >= 0) copy16(tok_base, tok_off[b][q] + koff, stage + tok_dst[b][q]);
+                if (tok_dst[b][q] >= 0) {
+                    if (tok_live[b][q]) copy16(tok_base, tok_off[b][q] + koff, stage + tok_dst[b][q]);
+                }
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -246,9 +252,37 @@ __device__ __forceinline__ void mma_fp8_step(f32x16 (&acc)[2][4], const char *to
 // FULL (RB = 64 only): the tile has two completely live blocks, so geometry and wait counts are
 // compile-time constants (`lay` must be that geometry); otherwise both are wave-uniform run-time
 // values and the wait count goes through a switch.
+//
+// Slab 0 goes to stage `stage0`, the following ones to the stages behind it (wrapping).  `n_pre`: the
+// caller has already issued slabs 0 .. n_pre - 1 (see pre_issue; a workgroup that runs one tile
+// after another issues them under the previous tile's epilogue).
+template <int DT, int RB, bool FULL>
+__device__ __forceinline__ int stage_bytes(const Layout &lay) {
+    return FULL ? FullCfg<DT>::kStageBytes : lay.stage_bytes;
+}
+template <int DT, int RB, bool FULL>
+__device__ __forceinline__ int stage_count(const Layout &lay) {
+    return FULL ? FullCfg<DT>::kStages : lay.stages;
+}
+// Issues slabs 0 .. n - 1 of a tile (at most stages - 1 of them, in rotated order from `start`) into
+// stages stage0, stage0 + 1, ...
+template <int DT, int RB, bool FULL>
+__device__ __forceinline__ void pre_issue(const Loader<RB> &ld, const Layout &lay, char *lds, int n_slabs, int start,
+                                          int stage0, int n) {
+    const int SB = stage_bytes<DT, RB, FULL>(lay), NS = stage_count<DT, RB, FULL>(lay);
+    for (int s = 0; s < n; ++s) {
+        if (s >= n_slabs) break;
+        int slab = s + start;
+        if (slab >= n_slabs) slab -= n_slabs;
+        int st = stage0 + s;
+        if (st >= NS) st -= NS;
+        ld.issue(lds + st * SB, slab);
+    }
+}
 template <int DT, int RB, int NTF, bool TRANSPOSED, bool COMPUTE, bool FULL>
 __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader<RB> &ld, const Layout &lay, char *lds,
-                                          int n_slabs, const int (&wrow)[2], int lane, int tok_region, int start) {
+                                          int n_slabs, const int (&wrow)[2], int lane, int tok_region, int start,
+                                          int stage0 = 0, int n_pre = 0) {
     static_assert(!FULL || RB == 64, "the constant geometry is the 64-byte one");
     using F = FullCfg<DT>;
     const int SB = FULL ? F::kStageBytes : lay.stage_bytes;
@@ -261,8 +295,11 @@ __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader<RB> 
         s += start;
         return s >= n_slabs ? s - n_slabs : s;
     };
-    for (int s = 0; s < NS - 1; ++s)
-        if (s < n_slabs) ld.issue(lds + s * SB, rot(s));
+    for (int s = n_pre; s < NS - 1; ++s) {
+        int st = stage0 + s;
+        if (st >= NS) st -= NS;
+        if (s < n_slabs) ld.issue(lds + st * SB, rot(s));
+    }
     FragsBf16 fx, fy;  // fy carries the held-back sub-step across the barrier
     if constexpr (DT == DT_BF16 && COMPUTE) {
 #pragma unroll
@@ -275,8 +312,9 @@ __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader<RB> 
             for (int i = 0; i < 8; ++i) fy.b[t][i] = (__bf16)0.0f;
     }
     const int lps = ld.lps;
-    int cur_off = 0;               // stage of slab kt
-    int fill_off = (NS - 1) * SB;  // stage slab kt + NS - 1 goes to (the one slab kt - 1 used)
+    int cur_off = stage0 * SB;  // stage of slab kt
+    // stage slab kt + NS - 1 goes to (the one slab kt - 1 used)
+    int fill_off = (stage0 == 0 ? NS - 1 : stage0 - 1) * SB;
     for (int kt = 0; kt < n_slabs; ++kt) {
         // slab kt has landed once at most the copies of the later slabs (up to NS - 2) are pending
         if constexpr (FULL) {

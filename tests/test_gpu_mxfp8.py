@@ -112,3 +112,34 @@ def test_validation_errors(device):
         call(xs=a["x_scales"][:, :4].contiguous())
     with pytest.raises(RuntimeError):
         call(w1s=a["w1_scales"].reshape(-1)[:-1].contiguous())
+
+
+@pytest.mark.parametrize("per", [2, 3, 16])
+@pytest.mark.parametrize("T,K,E,N,top_k", [
+    (300, 1280, 4, 1280, 2),   # wide tiles of every kind; 5 up and 5 down weight tiles (not a multiple of 2 or 3)
+    (24, 768, 6, 768, 3),      # tiles of one fragment: the down tile stores from registers
+])
+def test_several_weight_tiles_per_workgroup(T, K, E, N, top_k, per, device):
+    # a workgroup that walks `per` weight tiles with its token rows must give the bits of one tile per
+    # workgroup (same sums in the same order), and both must pass the oracle gates
+    import prime_moe
+    from prime_moe import _native
+    lib = _native.load()
+    g, a, deq = _quantised_inputs(T, K, E, N, device, seed=per)
+    ids, wts = reference_routing(T, E, top_k, device, g)
+    sched = torch.ops.prime_moe.moe_align(ids, E, 128, 1)
+    outs = []
+    try:
+        for n in (1, per):
+            lib.pmoe_set_tiles_per_workgroup(n)
+            out = torch.full((T, K), float("nan"), dtype=torch.bfloat16, device=device)
+            prime_moe.fused_moe_mxfp8(a["x"], a["x_scales"], a["w1"], a["w1_scales"], a["w2"], a["w2_scales"],
+                                      *sched, wts, out, top_k, 128, 64, 4, 2, 1, True)
+            torch.cuda.synchronize()
+            outs.append(out)
+    finally:
+        lib.pmoe_set_tiles_per_workgroup(0)
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    ref = O.fused_moe_dense(deq["x"], deq["w1"], deq["w2"], ids.cpu(), wts.cpu(), act_mx=True)
+    got = outs[1].float().cpu()
+    assert cosine(got, ref) >= MX_COS_GATE and rel_l2(got, ref) <= MX_RELL2_GATE

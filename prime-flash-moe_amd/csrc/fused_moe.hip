@@ -45,7 +45,8 @@ struct MoeArgs {
     int32_t *inv;         // (M * top_k): sorted row of each pair id (validated against sorted_ids when read)
     const int2 *tiles;    // row tiles built by the prologue: (first block, number of blocks 1..2)
     const int *n_tiles;   // number of row tiles
-    const int2 *work;     // this kernel's tile order: (first block | blocks << 28, weight tile)
+    const int4 *work;     // this kernel's work list, one entry per workgroup (see emit_work)
+    char *y_tail;         // partial tiles of down jobs whose contraction is split (see plan_tail_split)
     int top_k, M, K, N, H, E, sorted_num;
     int n_blocks;  // sorted_num / 128 (rounded up)
     int n_wtiles;  // weight tiles along the free dimension: H/128 (up) or ceil(K/256) (down)
@@ -63,17 +64,28 @@ constexpr int kPartRB = PMOE_PART_RB;      // of mxfp8 tiles with more, short of
 constexpr int kActPitchBf16 = 272;  // 128 bf16 + 16 B pad: 16-byte aligned rows, 2-way conflicts at most
 constexpr int kActPitchFp8 = 144;   // 128 e4m3 + 16 B pad
 
-// Workgroup id -> (first block, blocks, first weight tile, expert, number of weight tiles): one load
-// from the work list, which the prologue lays out by workgroup id (see emit_work); entries of
-// workgroups without work are -1.
-__device__ __forceinline__ bool resolve_tile(const MoeArgs &a, int &first, int &nb, int &wt, int &e, int &n_sub) {
-    const int2 w = a.work[blockIdx.x];
+// What one workgroup does: `n_sub` consecutive weight tiles from `wt` on for the row tile of `nb` blocks
+// starting at block `first`, expert `e`.  A down job can be one of `parts` workgroups that split the
+// contraction of one tile: this one sums slabs [part n / parts, (part + 1) n / parts) of the n; part 0
+// writes y, part p > 0 its own tile `slot + p - 1` of y_tail, and the finalize kernel adds them up.
+struct Job {
+    int first, nb, wt, e, n_sub;
+    int part, parts, slot;
+};
+
+// Workgroup id -> job: one load from the work list, which the prologue lays out by workgroup id (see
+// emit_work); entries of workgroups without work are -1.
+__device__ __forceinline__ bool resolve_job(const MoeArgs &a, Job &j) {
+    const int4 w = a.work[blockIdx.x];
     if (w.x < 0) return false;
-    first = w.x & 0x0fffffff;
-    nb = w.x >> 28;
-    wt = w.y & 0xffff;
-    e = (w.y >> 16) & 0x3ff;
-    n_sub = ((w.y >> 26) & 0xf) + 1;
+    j.first = w.x & 0x0fffffff;
+    j.nb = w.x >> 28;
+    j.wt = w.y & 0xffff;
+    j.e = (w.y >> 16) & 0x3ff;
+    j.n_sub = ((w.y >> 26) & 0xf) + 1;
+    j.part = w.z & 0xf;
+    j.parts = (w.z >> 4) & 0xf;
+    j.slot = w.z >> 8;
     return true;
 }
 
@@ -144,19 +156,38 @@ __device__ __forceinline__ void y_epilogue(const f32x16 (&acc)[2][4], char *tile
         }
     }
 }
+// Where a group's 128 x 256 output tile goes: y rows of the sorted order (row pitch K, the last tile of
+// a K that is not a multiple of 256 has 128 columns) or a tile of y_tail (256 x 256, pitch 512 bytes).
+struct YDst {
+    char *base;     // first row, first column of the group's tile
+    int64_t pitch;  // bytes per row
+    int cols;       // columns to write
+};
+__device__ __forceinline__ YDst y_destination(const MoeArgs &a, const Job &j, int grp, int k0) {
+    YDst d;
+    if (j.part == 0) {
+        d.base = a.y + (((int64_t)(j.first + grp) * kBlockRows) * a.K + k0) * 2;
+        d.pitch = (int64_t)a.K * 2;
+        d.cols = min(kWRows, a.K - k0);
+    } else {
+        d.base = a.y_tail + ((int64_t)(j.slot + j.part - 1) * 2 + grp) * (kBlockRows * kWRows * 2);
+        d.pitch = kWRows * 2;
+        d.cols = kWRows;
+    }
+    return d;
+}
 // Tiles with a single live fragment skip the detour through LDS: every lane stores its 8-byte runs
-// straight to y (32 rows x 16 KB per tile at most; a barrier and an LDS round trip cost more).
-__device__ __forceinline__ void store_y_direct(const MoeArgs &a, const f32x16 (&acc)[2][4], int64_t row0, int k0,
-                                               int n_rows, int w4, int lane) {
+// straight to the destination (32 rows x 16 KB per tile at most; a barrier and an LDS round trip cost more).
+__device__ __forceinline__ void store_y_direct(const YDst &d, const f32x16 (&acc)[2][4], int n_rows, int w4, int lane) {
     const int r = lane & 31, half = lane >> 5;
     if (r >= n_rows) return;
-    char *dst = a.y + ((row0 + r) * a.K + k0) * 2;
+    char *dst = d.base + r * d.pitch;
 #pragma unroll
     for (int f = 0; f < 2; ++f)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const int col = 64 * w4 + 32 * f + 8 * g + 4 * half;
-            if (k0 + col < a.K) {
+            if (col < d.cols) {
                 uint2 pk;
                 pk.x = pack2_bf16(acc[f][0][4 * g], acc[f][0][4 * g + 1]);
                 pk.y = pack2_bf16(acc[f][0][4 * g + 2], acc[f][0][4 * g + 3]);
@@ -164,18 +195,16 @@ __device__ __forceinline__ void store_y_direct(const MoeArgs &a, const f32x16 (&
             }
         }
 }
-// ... and its first n_rows rows are copied to y rows row0.., columns [k0, k0 + 256) (the last
-// tile of a K that is not a multiple of 256 has 128 columns); gt = thread index inside the group.
-__device__ __forceinline__ void store_y_tile(const MoeArgs &a, const char *tile, int64_t row0, int k0, int n_rows, int gt) {
-    const int K = a.K;
+// ... and its first n_rows rows are copied to the destination; gt = thread index inside the group.
+__device__ __forceinline__ void store_y_tile(const YDst &d, const char *tile, int n_rows, int gt) {
     const int c = gt & 31;
-    if (k0 + 8 * c >= K) return;
+    if (8 * c >= d.cols) return;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int row = (gt >> 5) + 8 * i;
         if (row < n_rows) {
             const uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kYPitch + c * 16);
-            *reinterpret_cast<uint4 *>(a.y + ((row0 + row) * K + k0) * 2 + c * 16) = v;
+            *reinterpret_cast<uint4 *>(d.base + row * d.pitch + c * 16) = v;
         }
     }
 }
@@ -467,8 +496,9 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
     using L = SplitLds<DT>;
     __shared__ __attribute__((aligned(1024))) char lds[L::kTotal];
     RowInfo<2> &ri = *reinterpret_cast<RowInfo<2> *>(lds + L::kRowInfoOff);
-    int first, nb, ht, e, n_sub;
-    if (!resolve_tile(a, first, nb, ht, e, n_sub)) return;
+    Job j;
+    if (!resolve_job(a, j)) return;
+    const int first = j.first, nb = j.nb, ht = j.wt, e = j.e, n_sub = j.n_sub;
     const int ntf = load_row_info<2>(a, first, nb, ri);
     if (ntf == 0) return;
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
@@ -490,9 +520,9 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
 // Down kernel of the split pipeline: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
 // full reduction over H inside the workgroup (no split-K), then w[row] * y added to accum[token].
 template <int DT, int RB, int NTF, bool FULL>
-__device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int kt, int n_sub, int e, RowInfo<2> &ri,
-                                               char *lds) {
+__device__ __forceinline__ void down_tile_ring(const MoeArgs &a, const Job &job, RowInfo<2> &ri, char *lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
+    const int first = job.first, kt = job.wt, n_sub = job.n_sub, e = job.e;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
     const int K = a.K, H = a.H;
@@ -507,12 +537,17 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
     int k0 = kt * kWRows;
     const uint32_t row_bytes = (uint32_t)(H * ES);
     const int hb = H >> 5, ht128 = H >> 7;
+    // this workgroup's share of the contraction (all of it unless the tile is split, which only
+    // happens to bf16 tiles: the scales of a slab are addressed from the start of the row)
+    const int n_slabs_all = (H * ES) / RB;
+    const int slab0 = job.part * n_slabs_all / job.parts;
+    const int n_slabs = (job.part + 1) * n_slabs_all / job.parts - slab0;
     ring::Loader<RB> ld;
-    ld.tok_base = a.act + row0 * H * ES;
+    ld.tok_base = a.act + row0 * H * ES + slab0 * RB;
     // weight rows (output columns) k0 .. k0 + 255 of the expert; the last tile of a K that is not a
     // multiple of 256 has 128 of them and reads the first half twice
     auto set_weights = [&](int k) {
-        ld.w_base[0] = a.w2 + ((int64_t)e * K + k) * H * ES;
+        ld.w_base[0] = a.w2 + ((int64_t)e * K + k) * H * ES + slab0 * RB;
         ld.w_base[1] = (k + 128 < K) ? ld.w_base[0] + (int64_t)128 * H * ES : ld.w_base[0];
         if (DT == DT_FP8 && wave >= 4)
             ld.sc_off = (uint32_t)blocked_scale_off(min(k + 64 * (wave - 4) + lane, K - 1), 0, ht128);
@@ -526,7 +561,6 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
         [&](int row) { return (uint32_t)blocked_scale_off(min(k0 + row, K - 1), 0, ht128); });
 
     const int wrow[2] = {64 * w4, 64 * w4 + 32};
-    const int n_slabs = (H * ES) / RB;
     const int start = slab_rotation<RB>(n_slabs);
     const int tok_region = grp ? lay.group1_off : 0;
     const int SB = ring::stage_bytes<DT, RB, FULL>(lay), NS = ring::stage_count<DT, RB, FULL>(lay);
@@ -551,13 +585,14 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
             n_pre = free0 < NS ? min(NS - 1, NS - free0) : 0;
             ring::pre_issue<DT, RB, FULL>(ld, lay, lds, n_slabs, start, stage0, n_pre);
         }
+        const YDst dst = y_destination(a, job, grp, k0);
         if constexpr (NTF == 1) {
-            if (active) store_y_direct(a, acc, row0 + grp * kBlockRows, k0, my_rows, w4, lane);
+            if (active) store_y_direct(dst, acc, my_rows, w4, lane);
         } else {
             char *tile = lds + grp * (kBlockRows * kYPitch);
             if (active) y_epilogue<NTF>(acc, tile, w4, lane);
             __syncthreads();
-            if (active) store_y_tile(a, tile, row0 + grp * kBlockRows, k0, my_rows, gt);
+            if (active) store_y_tile(dst, tile, my_rows, gt);
             if (more) __syncthreads();  // the tiles have been read: the head of the ring may be filled again
         }
         k0 += kWRows;
@@ -566,7 +601,8 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, int first, int 
 
 // Down kernel tile on the 128-byte unit ring (bf16).
 template <int NTF>
-__device__ __forceinline__ void down_tile_wide_bf16(const MoeArgs &a, int first, int kt, int e, RowInfo<2> &ri, char *lds) {
+__device__ __forceinline__ void down_tile_wide_bf16(const MoeArgs &a, const Job &job, RowInfo<2> &ri, char *lds) {
+    const int first = job.first, kt = job.wt, e = job.e;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
     const int K = a.K, H = a.H;
@@ -579,27 +615,31 @@ __device__ __forceinline__ void down_tile_wide_bf16(const MoeArgs &a, int first,
     const bool active = my_ntf > 0;
 
     const uint32_t row_bytes = (uint32_t)H * 2u;
-    const char *w_lo = a.w2 + ((int64_t)e * K + k0) * H * 2;
+    // this workgroup's share of the contraction (all of it unless the tile is split)
+    const int n_slabs_all = (int)(row_bytes / ring128::kRB);
+    const int slab0 = job.part * n_slabs_all / job.parts;
+    const int n_slabs = (job.part + 1) * n_slabs_all / job.parts - slab0;
+    const char *w_lo = a.w2 + ((int64_t)e * K + k0) * H * 2 + slab0 * ring128::kRB;
     const char *w_hi = (k0 + 128 < K) ? w_lo + (int64_t)128 * H * 2 : w_lo;
     ring128::Loader ld;
-    ld.setup(tid, a.act + row0 * H * 2, w_lo, w_hi, row_bytes, ntf0, ntf1,
+    ld.setup(tid, a.act + row0 * H * 2 + slab0 * ring128::kRB, w_lo, w_hi, row_bytes, ntf0, ntf1,
              [&](int row) { return (uint32_t)row * row_bytes; });
 
     const int wrow[2] = {64 * w4, 64 * w4 + 32};
     f32x16 acc[2][4];
     zero_acc(acc);
-    const int n_slabs = (int)(row_bytes / ring128::kRB);
     const int start = slab_rotation128(n_slabs);
     const int tok_region = grp * ring128::kGroupRegion;
     if (active) ring128::main_loop<NTF, true, true>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
     else ring128::main_loop<NTF, true, false>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
+    const YDst dst = y_destination(a, job, grp, k0);
     if constexpr (NTF == 1) {
-        if (active) store_y_direct(a, acc, row0 + grp * kBlockRows, k0, my_rows, w4, lane);
+        if (active) store_y_direct(dst, acc, my_rows, w4, lane);
     } else {
         char *tile = lds + grp * (kBlockRows * kYPitch);
         if (active) y_epilogue<NTF>(acc, tile, w4, lane);
         __syncthreads();
-        if (active) store_y_tile(a, tile, row0 + grp * kBlockRows, k0, my_rows, gt);
+        if (active) store_y_tile(dst, tile, my_rows, gt);
     }
 }
 
@@ -608,22 +648,23 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
     using L = SplitLds<DT>;
     __shared__ __attribute__((aligned(1024))) char lds[L::kTotal];
     RowInfo<2> &ri = *reinterpret_cast<RowInfo<2> *>(lds + L::kRowInfoOff);
-    int first, nb, kt, e, n_sub;
-    if (!resolve_tile(a, first, nb, kt, e, n_sub)) return;
-    const int ntf = load_row_info<2>(a, first, nb, ri);
+    Job j;
+    if (!resolve_job(a, j)) return;
+    const int ntf = load_row_info<2>(a, j.first, j.nb, ri);
     if (ntf == 0) return;
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {  // one weight tile per workgroup on this path (see launch_pipeline)
-        if (skinny) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, 1, e, ri, lds);
-        else if (ntf == 1) down_tile_wide_bf16<1>(a, first, kt, e, ri, lds);
-        else if (ntf == 2) down_tile_wide_bf16<2>(a, first, kt, e, ri, lds);
-        else down_tile_wide_bf16<4>(a, first, kt, e, ri, lds);
+        j.n_sub = 1;
+        if (skinny) down_tile_ring<DT, kSkinnyRB, 1, false>(a, j, ri, lds);
+        else if (ntf == 1) down_tile_wide_bf16<1>(a, j, ri, lds);
+        else if (ntf == 2) down_tile_wide_bf16<2>(a, j, ri, lds);
+        else down_tile_wide_bf16<4>(a, j, ri, lds);
     } else {
         const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-        if (ntf == 1) down_tile_ring<DT, kSkinnyRB, 1, false>(a, first, kt, n_sub, e, ri, lds);
-        else if (ntf == 2) down_tile_ring<DT, kPartRB, 2, false>(a, first, kt, n_sub, e, ri, lds);
-        else if (full) down_tile_ring<DT, 64, 4, true>(a, first, kt, n_sub, e, ri, lds);
-        else down_tile_ring<DT, kPartRB, 4, false>(a, first, kt, n_sub, e, ri, lds);
+        if (ntf == 1) down_tile_ring<DT, kSkinnyRB, 1, false>(a, j, ri, lds);
+        else if (ntf == 2) down_tile_ring<DT, kPartRB, 2, false>(a, j, ri, lds);
+        else if (full) down_tile_ring<DT, 64, 4, true>(a, j, ri, lds);
+        else down_tile_ring<DT, kPartRB, 4, false>(a, j, ri, lds);
     }
 }
 
@@ -635,10 +676,40 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
 // more workgroups then ask for the same lines at the same moment.)
 // Hardware hands consecutive workgroup ids to the 8 XCDs round-robin, so position `l` of the walk
 // is given to workgroup id 8 * (l mod per_xcd) + l / per_xcd: one XCD then runs a contiguous range of
-// the walk.  The entry carries everything the workgroup needs to start: (first block | blocks << 28,
-// first weight tile | expert << 16 | (weight tiles - 1) << 26); experts < 1024, up to 16 weight tiles.
-__device__ __forceinline__ void emit_work(int2 *work, int n_wt, int per_job, int tile, int n_tiles, int first, int nb,
-                                          int e) {
+// the walk.  The entry carries everything the workgroup needs to start: x = first block | blocks << 28,
+// y = first weight tile | expert << 16 | (weight tiles - 1) << 26 (experts < 1024, up to 16 weight
+// tiles), z = part | parts << 4 | tail slot << 8 (see TailSplit).
+//
+// Workgroups start in the order of their ids, so the last `per_xcd_tail` positions of every XCD's range
+// are the jobs that would run while most CUs have nothing left to do.  The down kernel splits the
+// contraction of each of them over `parts` workgroups: part 0 stays in place, the others go behind the
+// list proper (from entry `extra_base` on) and write partial tiles to y_tail, which the finalize
+// kernel adds (tail_tab tells it which tiles have parts and where).
+constexpr int kTailSlots = 192;  // partial tiles y_tail holds (256 x 256 bf16 each)
+struct TailSplit {
+    int parts;         // 1: no split
+    int per_xcd_tail;  // jobs split at the end of each XCD's range
+    int extra_base;    // first work list entry of the parts > 0
+    int *tail_tab;     // per (block, weight tile): 0, or first slot << 8 | block inside its tile << 4 | parts
+};
+
+// How the tail of `n_jobs` down jobs on `n_cus` CUs is split; every part gets at least one slab.
+__device__ __forceinline__ void plan_tail_split(TailSplit &ts, int n_jobs, int n_cus, int n_slabs) {
+    ts.parts = 1;
+    ts.per_xcd_tail = 0;
+    if (n_cus <= 0 || n_jobs <= 0) return;
+    const int rounds = n_jobs / n_cus, rest = n_jobs % n_cus;
+    if (rest == 0 || rounds >= 16) return;  // nothing left over, or too little to matter
+    int parts = min(min(4, n_slabs), n_cus / rest);
+    const int per_xcd_tail = (rest + 7) >> 3;
+    while (parts > 1 && per_xcd_tail * 8 * (parts - 1) > kTailSlots) --parts;
+    if (parts < 2) return;
+    ts.parts = parts;
+    ts.per_xcd_tail = per_xcd_tail;
+}
+
+__device__ __forceinline__ void emit_work(int4 *work, int n_wt, int per_job, int tile, int n_tiles, int first, int nb,
+                                          int e, const TailSplit *ts) {
     constexpr int GW = 8;
     const int n_jobs = (n_wt + per_job - 1) / per_job;  // a workgroup takes `per_job` consecutive weight tiles
     const int per_xcd = (n_tiles * n_jobs + 7) >> 3;
@@ -647,7 +718,17 @@ __device__ __forceinline__ void emit_work(int2 *work, int n_wt, int per_job, int
         const int gw = min(GW, n_jobs - wg * GW);
         const int l = wg * GW * n_tiles + tile * gw + (j - wg * GW);
         const int wt = j * per_job, cnt = min(per_job, n_wt - wt);
-        work[8 * (l % per_xcd) + l / per_xcd] = make_int2(first | (nb << 28), wt | (e << 16) | ((cnt - 1) << 26));
+        const int x = first | (nb << 28), y = wt | (e << 16) | ((cnt - 1) << 26);
+        const int pos = l % per_xcd, xcd = l / per_xcd;
+        if (ts != nullptr && ts->parts > 1 && pos >= per_xcd - ts->per_xcd_tail) {
+            const int slot = ((pos - (per_xcd - ts->per_xcd_tail)) * 8 + xcd) * (ts->parts - 1);
+            const int z = (ts->parts << 4) | (slot << 8);
+            work[8 * pos + xcd] = make_int4(x, y, z, 0);
+            for (int p = 1; p < ts->parts; ++p) work[ts->extra_base + slot + p - 1] = make_int4(x, y, z | p, 0);
+            for (int b = 0; b < nb; ++b) ts->tail_tab[(first + b) * n_wt + wt] = (slot << 8) | (b << 4) | ts->parts;
+        } else {
+            work[8 * pos + xcd] = make_int4(x, y, 1 << 4, 0);
+        }
     }
 }
 
@@ -658,17 +739,20 @@ __device__ __forceinline__ void emit_work(int2 *work, int n_wt, int per_job, int
 // in the schedule keep whatever the buffer held; the reader validates an entry against sorted_ids.
 __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert_ids, const int32_t *ntpp,
                                                            int n_blocks, int2 *tiles, int *n_tiles,
-                                                           int2 *work_up, int n_wt_up, int per_job_up, int grid_up,
-                                                           int2 *work_down, int n_wt_down, int per_job_down,
-                                                           int grid_down, int num_experts,
+                                                           int4 *work_up, int n_wt_up, int per_job_up, int grid_up,
+                                                           int4 *work_down, int n_wt_down, int per_job_down,
+                                                           int grid_down, int split_cus, int down_slabs,
+                                                           int *tail_tab, int num_experts,
                                                            const int32_t *sorted_ids, int sorted_num, int32_t *inv,
                                                            int n_pairs, int do_invert, const uint8_t *x_scales,
                                                            uint32_t *xs_tiled, int nkt, int top_k, int M) {
     if (blockIdx.x == 0 && tiles != nullptr) {
         __shared__ int s_max[4], s_sum[4], s_carry[2];
         const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-        for (int i = tid; i < grid_up; i += 256) work_up[i] = make_int2(-1, -1);
-        for (int i = tid; i < grid_down; i += 256) work_down[i] = make_int2(-1, -1);
+        for (int i = tid; i < grid_up; i += 256) work_up[i] = make_int4(-1, -1, 0, 0);
+        for (int i = tid; i < grid_down; i += 256) work_down[i] = make_int4(-1, -1, 0, 0);
+        if (tail_tab != nullptr)
+            for (int i = tid; i < n_blocks * n_wt_down; i += 256) tail_tab[i] = 0;
         const int n_live = min((ntpp[0] + kBlockRows - 1) / kBlockRows, n_blocks);
         if (tid == 0) { s_carry[0] = 0; s_carry[1] = 0; }
         __syncthreads();
@@ -709,12 +793,17 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
         if (tid == 0) n_tiles[0] = nt;
         __threadfence_block();
         __syncthreads();  // tiles written above are read below by other threads
+        TailSplit ts;
+        ts.extra_base = grid_down - kTailSlots;
+        ts.tail_tab = tail_tab;
+        plan_tail_split(ts, tail_tab != nullptr ? nt * ((n_wt_down + per_job_down - 1) / per_job_down) : 0, split_cus,
+                        down_slabs);
         for (int t = tid; t < nt; t += 256) {
             const int2 tl = tiles[t];
             const int e = expert_ids[tl.x];
             if (e < 0 || e >= num_experts) continue;  // nothing to compute for a block without an expert
-            emit_work(work_up, n_wt_up, per_job_up, t, nt, tl.x, tl.y, e);
-            emit_work(work_down, n_wt_down, per_job_down, t, nt, tl.x, tl.y, e);
+            emit_work(work_up, n_wt_up, per_job_up, t, nt, tl.x, tl.y, e, nullptr);
+            emit_work(work_down, n_wt_down, per_job_down, t, nt, tl.x, tl.y, e, &ts);
         }
     }
     if (do_invert) {
@@ -765,12 +854,14 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
 }
 
 // out[t, 8 columns] = bf16(sum over the token's top_k pairs p, in pair order, of w[p] * y[row(p)])
+// (y[row] = the row's part 0 plus, for tiles the down kernel split, the partial rows in y_tail)
 // (ACCUMULATE: added to what `out` holds).  row(p) = inv[p] if that row really holds p, else the
 // pair was dropped by the schedule and contributes nothing.  One thread per (token, 8 columns).
 template <bool ACCUMULATE>
 __global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int32_t *inv, const int32_t *sorted_ids,
                                                        const int32_t *ntpp, int sorted_num, const float *topk_w,
-                                                       int top_k, int M, int K, uint4 *out) {
+                                                       int top_k, int M, int K, uint4 *out, const int *tail_tab,
+                                                       const char *y_tail, int n_wt) {
     const int k8 = K >> 3;
     const int64_t total = (int64_t)M * k8;
     const int n_rows = min(ntpp[0], sorted_num);
@@ -783,12 +874,21 @@ __global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int3
             const int row = inv[p];
             if (row < 0 || row >= n_rows || sorted_ids[row] != p) continue;
             const float w = topk_w[p];
-            const uint4 q = *reinterpret_cast<const uint4 *>(y + ((int64_t)row * K + 8 * c) * 2);
-            const uint32_t u[4] = {q.x, q.y, q.z, q.w};
+            auto add = [&](const uint4 q) {
+                const uint32_t u[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                v[2 * j] += w * bf16_bits_to_f32(u[j] & 0xffffu);
-                v[2 * j + 1] += w * bf16_bits_to_f32(u[j] >> 16);
+                for (int j = 0; j < 4; ++j) {
+                    v[2 * j] += w * bf16_bits_to_f32(u[j] & 0xffffu);
+                    v[2 * j + 1] += w * bf16_bits_to_f32(u[j] >> 16);
+                }
+            };
+            add(*reinterpret_cast<const uint4 *>(y + ((int64_t)row * K + 8 * c) * 2));
+            // a tile whose contraction was split: the other parts' partial rows, in part order
+            const int tt = tail_tab != nullptr ? tail_tab[(row >> 7) * n_wt + (c >> 5)] : 0;
+            if (tt != 0) {
+                const int parts = tt & 15, rr = ((tt >> 4) & 15) * kBlockRows + (row & 127), slot = tt >> 8;
+                for (int part = 1; part < parts; ++part)
+                    add(*reinterpret_cast<const uint4 *>(y_tail + (((int64_t)(slot + part - 1) * 256 + rr) * 256 + 8 * (c & 31)) * 2));
             }
         }
         uint32_t o[4];
@@ -810,7 +910,8 @@ __global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int3
 // ------------------------------------------------------------------------------------------ host
 
 struct WorkspaceLayout {
-    size_t n_tiles_off, tiles_off, work_up_off, work_down_off, inv_off, y_off, act_off, act_scales_off, xs_tiled_off, total;
+    size_t n_tiles_off, tiles_off, work_up_off, work_down_off, tail_tab_off, y_tail_off, inv_off, y_off, act_off,
+        act_scales_off, xs_tiled_off, total;
 };
 
 static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_num, int top_k) {
@@ -824,9 +925,14 @@ static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_
     l.tiles_off = off;
     off = align_up(off + blocks * sizeof(int2), 256);
     l.work_up_off = off;
-    off = align_up(off + blocks * (H / 128) * sizeof(int2), 256);
+    off = align_up(off + align_up(blocks * (H / 128), 8) * sizeof(int4), 256);
     l.work_down_off = off;
-    off = align_up(off + blocks * (((size_t)K + kWRows - 1) / kWRows) * sizeof(int2), 256);
+    const size_t n_wt_down = ((size_t)K + kWRows - 1) / kWRows;
+    off = align_up(off + (align_up(blocks * n_wt_down, 8) + kTailSlots) * sizeof(int4), 256);
+    l.tail_tab_off = off;
+    if (dt == DT_BF16) off = align_up(off + blocks * n_wt_down * sizeof(int32_t), 256);
+    l.y_tail_off = off;
+    if (dt == DT_BF16) off = align_up(off + (size_t)kTailSlots * kWRows * kWRows * 2, 256);
     l.inv_off = off;
     off = align_up(off + (size_t)M * (size_t)std::max(top_k, 1) * sizeof(int32_t), 256);
     l.y_off = off;
@@ -880,8 +986,9 @@ static int tiles_per_workgroup(int dt, bool down, int n_blocks, int n_wt) {
 struct SchedBuffers {
     int2 *tiles;
     int *n_tiles;
-    int2 *work_up;
-    int2 *work_down;
+    int4 *work_up;
+    int4 *work_down;
+    int *tail_tab;  // null: the down kernel's tail is not split (mxfp8)
 };
 
 template <int DT>
@@ -896,14 +1003,15 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
     const int per_up = tiles_per_workgroup(DT, false, a.n_blocks, a.n_wtiles);
     const int per_down = tiles_per_workgroup(DT, true, a.n_blocks, n_wt_down);
     const int grid_up = grid_for(a.n_blocks * ((a.n_wtiles + per_up - 1) / per_up));
-    const int grid_down = grid_for(a.n_blocks * ((n_wt_down + per_down - 1) / per_down));
+    // the parts > 0 of split tail jobs sit behind the list proper
+    const int grid_down = grid_for(a.n_blocks * ((n_wt_down + per_down - 1) / per_down)) + kTailSlots;
     {
         // the work lists are needed by the two kernels even when the rest of the prologue is masked off
         const int do_invert = (mask & PMOE_PHASE_PROLOGUE) ? 1 : 0;
         const int blocks = do_invert ? std::max(1, std::min((a.sorted_num + 255) / 256, 1024)) : 1;
         hipLaunchKernelGGL(moe_prologue_kernel, dim3(blocks), dim3(256), 0, s, a.expert_ids, a.ntpp, a.n_blocks,
                            sb.tiles, sb.n_tiles, sb.work_up, a.n_wtiles, per_up, grid_up,
-                           sb.work_down, n_wt_down, per_down, grid_down, a.E,
+                           sb.work_down, n_wt_down, per_down, grid_down, resident_grid(), a.H * 2 / 128, sb.tail_tab, a.E,
                            a.sorted_ids, a.sorted_num, a.inv, a.M * a.top_k, do_invert, a.x_scales, a.xs_tiled,
                            a.K >> 7, a.top_k, a.M);
     }
@@ -922,10 +1030,12 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
         const int blocks = (int)std::min<int64_t>((n8 + 255) / 256, 8192);
         if (split)
             hipLaunchKernelGGL(finalize_kernel<false>, dim3(blocks), dim3(256), 0, s, a.y, a.inv, a.sorted_ids, a.ntpp,
-                               a.sorted_num, a.topk_w, a.top_k, a.M, a.K, reinterpret_cast<uint4 *>(out));
+                               a.sorted_num, a.topk_w, a.top_k, a.M, a.K, reinterpret_cast<uint4 *>(out), sb.tail_tab,
+                               a.y_tail, n_wt_down);
         else
             hipLaunchKernelGGL(finalize_kernel<true>, dim3(blocks), dim3(256), 0, s, a.y, a.inv, a.sorted_ids, a.ntpp,
-                               a.sorted_num, a.topk_w, a.top_k, a.M, a.K, reinterpret_cast<uint4 *>(out));
+                               a.sorted_num, a.topk_w, a.top_k, a.M, a.K, reinterpret_cast<uint4 *>(out), sb.tail_tab,
+                               a.y_tail, n_wt_down);
     }
     return check_launch("fused_moe launch");
 }
@@ -934,8 +1044,9 @@ static SchedBuffers sched_buffers(char *ws, const WorkspaceLayout &l) {
     SchedBuffers sb;
     sb.n_tiles = reinterpret_cast<int *>(ws + l.n_tiles_off);
     sb.tiles = reinterpret_cast<int2 *>(ws + l.tiles_off);
-    sb.work_up = reinterpret_cast<int2 *>(ws + l.work_up_off);
-    sb.work_down = reinterpret_cast<int2 *>(ws + l.work_down_off);
+    sb.work_up = reinterpret_cast<int4 *>(ws + l.work_up_off);
+    sb.work_down = reinterpret_cast<int4 *>(ws + l.work_down_off);
+    sb.tail_tab = l.y_tail_off > l.tail_tab_off ? reinterpret_cast<int *>(ws + l.tail_tab_off) : nullptr;
     return sb;
 }
 
@@ -998,6 +1109,7 @@ extern "C" int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2,
     a.topk_w = topk_weights;
     char *ws = static_cast<char *>(workspace);
     a.y = ws + l.y_off;
+    a.y_tail = ws + l.y_tail_off;
     a.inv = reinterpret_cast<int32_t *>(ws + l.inv_off);
     a.act = ws + l.act_off;
     a.top_k = top_k; a.M = M; a.K = K; a.N = N; a.H = N / 2; a.E = num_experts; a.sorted_num = sorted_num;

@@ -47,6 +47,8 @@ struct MoeArgs {
     const int *n_tiles;   // number of row tiles
     const int4 *work;     // this kernel's work list, one entry per workgroup (see emit_work)
     char *y_tail;         // partial tiles of down jobs whose contraction is split (see plan_tail_split)
+    float *up_partials;   // fp32 partial accumulators of up jobs whose contraction is split
+    int *up_counters;     // per such job: parts that have stored theirs (zeroed by the prologue)
     int top_k, M, K, N, H, E, sorted_num;
     int n_blocks;  // sorted_num / 128 (rounded up)
     int n_wtiles;  // weight tiles along the free dimension: H/128 (up) or ceil(K/256) (down)
@@ -65,9 +67,12 @@ constexpr int kActPitchBf16 = 272;  // 128 bf16 + 16 B pad: 16-byte aligned rows
 constexpr int kActPitchFp8 = 144;   // 128 e4m3 + 16 B pad
 
 // What one workgroup does: `n_sub` consecutive weight tiles from `wt` on for the row tile of `nb` blocks
-// starting at block `first`, expert `e`.  A down job can be one of `parts` workgroups that split the
-// contraction of one tile: this one sums slabs [part n / parts, (part + 1) n / parts) of the n; part 0
-// writes y, part p > 0 its own tile `slot + p - 1` of y_tail, and the finalize kernel adds them up.
+// starting at block `first`, expert `e`.  A job of a bf16 kernel can be one of `parts` workgroups that
+// split the contraction of one tile (tail job number `slot`): this one sums slabs
+// [part n / parts, (part + 1) n / parts) of the n.  Down kernel: part 0 writes y, part p > 0 tile
+// slot (parts - 1) + p - 1 of y_tail, and the finalize kernel adds them up.  Up kernel: every part
+// stores its fp32 accumulators, and the one that finishes last adds them in part order and goes on to
+// the epilogue (see join_parts).
 struct Job {
     int first, nb, wt, e, n_sub;
     int part, parts, slot;
@@ -170,7 +175,7 @@ __device__ __forceinline__ YDst y_destination(const MoeArgs &a, const Job &j, in
         d.pitch = (int64_t)a.K * 2;
         d.cols = min(kWRows, a.K - k0);
     } else {
-        d.base = a.y_tail + ((int64_t)(j.slot + j.part - 1) * 2 + grp) * (kBlockRows * kWRows * 2);
+        d.base = a.y_tail + ((int64_t)(j.slot * (j.parts - 1) + j.part - 1) * 2 + grp) * (kBlockRows * kWRows * 2);
         d.pitch = kWRows * 2;
         d.cols = kWRows;
     }
@@ -287,6 +292,48 @@ __device__ __forceinline__ void store_act_tile(const MoeArgs &a, const char *til
     }
 }
 
+// Contraction split of an up tile: every part stores its accumulators (32 float4 per thread, thread
+// index fastest), makes them visible to the device and counts itself in; the part that counts last
+// adds all parts in part order (its own too, from memory: the same bits whichever part is last) and
+// returns true.  Nobody waits for anybody.  `lds_flag` is a word of LDS no copy is in flight to.
+constexpr int kUpTailJobs = 64;
+__device__ __forceinline__ bool join_parts(const MoeArgs &a, const Job &j, f32x16 (&acc)[2][4], int *lds_flag) {
+    const int tid = threadIdx.x;
+    float4 *mine = reinterpret_cast<float4 *>(a.up_partials) + ((int64_t)(j.slot * 4 + j.part) * 32) * 512;
+#pragma unroll
+    for (int f = 0; f < 2; ++f)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                mine[((f * 4 + t) * 4 + q) * 512 + tid] =
+                    make_float4(acc[f][t][4 * q], acc[f][t][4 * q + 1], acc[f][t][4 * q + 2], acc[f][t][4 * q + 3]);
+    __threadfence();  // the stores above are visible device-wide before the count below
+    __syncthreads();
+    if (tid == 0) *lds_flag = atomicAdd(&a.up_counters[j.slot], 1);
+    __syncthreads();
+    const bool last = *lds_flag == j.parts - 1;
+    if (!last) return false;
+    __threadfence();  // the other parts' stores are visible to the loads below
+    zero_acc(acc);
+    for (int p = 0; p < j.parts; ++p) {
+        const float4 *src = reinterpret_cast<const float4 *>(a.up_partials) + ((int64_t)(j.slot * 4 + p) * 32) * 512;
+#pragma unroll
+        for (int f = 0; f < 2; ++f)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 v = src[((f * 4 + t) * 4 + q) * 512 + tid];
+                    acc[f][t][4 * q] += v.x;
+                    acc[f][t][4 * q + 1] += v.y;
+                    acc[f][t][4 * q + 2] += v.z;
+                    acc[f][t][4 * q + 3] += v.w;
+                }
+    }
+    return true;
+}
+
 // ==========================================================================================
 // Two-group kernels on the ring engines
 // ==========================================================================================
@@ -373,9 +420,10 @@ __device__ __forceinline__ int slab_rotation(int n_slabs) {
 // wave v of a group owns gate/up rows 32v..32v+31 so gate and up of one activation element sit in the
 // same lane and register.
 template <int DT, int RB, int NTF, bool FULL>
-__device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht, int n_sub, int e, RowInfo<2> &ri,
-                                             char *lds, uint32_t *act_sc_lds) {
+__device__ __forceinline__ void up_tile_ring(const MoeArgs &a, const Job &job, RowInfo<2> &ri, char *lds,
+                                             uint32_t *act_sc_lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
+    const int first = job.first, ht = job.wt, n_sub = job.n_sub, e = job.e;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
     const int K = a.K, H = a.H, N = a.N;
@@ -386,9 +434,14 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
     const ring::Layout lay = ring::make_layout<DT, RB>(ntf0, ntf1, ring::ring_bytes<DT>());
 
     int h0 = ht * 128;
+    // this workgroup's share of the contraction (all of it unless the tile is split, which only
+    // happens to bf16 tiles: the scales of a slab are addressed from the start of the row)
+    const int n_slabs_all = (K * ES) / RB;
+    const int slab0 = job.part * n_slabs_all / job.parts;
+    const int n_slabs = (job.part + 1) * n_slabs_all / job.parts - slab0;
     ring::Loader<RB> ld;
-    ld.tok_base = a.x;
-    ld.w_base[0] = a.w1 + ((int64_t)e * N + h0) * K * ES;
+    ld.tok_base = a.x + slab0 * RB;
+    ld.w_base[0] = a.w1 + ((int64_t)e * N + h0) * K * ES + slab0 * RB;
     ld.w_base[1] = ld.w_base[0] + (int64_t)H * K * ES;
     const uint32_t row_bytes = (uint32_t)(K * ES);
     const int kb = K >> 5, kt128 = K >> 7;
@@ -401,7 +454,6 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
         [&](int row) { return (uint32_t)blocked_scale_off((row < 128 ? h0 : H + h0 - 128) + row, 0, K >> 7); });
 
     const int wrow[2] = {32 * w4, 128 + 32 * w4};
-    const int n_slabs = (K * ES) / RB;
     const int start = slab_rotation<RB>(n_slabs);
     const int tok_region = grp ? lay.group1_off : 0;
     // the ring is free after main_loop (it ends with a barrier): its head holds the activation tiles
@@ -421,6 +473,9 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, int first, int ht
             ring::main_loop<DT, RB, NTF, true, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
         else
             ring::main_loop<DT, RB, NTF, true, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
+        if constexpr (DT == DT_BF16) {
+            if (job.parts > 1 && !join_parts(a, job, acc, reinterpret_cast<int *>(lds + 128 * 1024))) return;
+        }
         const bool more = sub + 1 < n_sub;
         if (more) {
             // same token rows, the next 128 gate and 128 up rows of the expert
@@ -459,8 +514,9 @@ struct SplitLds {
 __device__ __forceinline__ int slab_rotation128(int n_slabs) { return (int)((blockIdx.x >> 3) & 7) % n_slabs; }
 
 // Up kernel tile on the 128-byte ring (bf16, two blocks or one block with more than 32 live rows).
-template <int NTF>
-__device__ __forceinline__ void up_tile_wide_bf16(const MoeArgs &a, int first, int ht, int e, RowInfo<2> &ri, char *lds) {
+template <int NTF, bool SPLIT>
+__device__ __forceinline__ void up_tile_wide_bf16(const MoeArgs &a, const Job &job, RowInfo<2> &ri, char *lds) {
+    const int first = job.first, ht = job.wt, e = job.e;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
     const int K = a.K, H = a.H, N = a.N;
@@ -471,19 +527,25 @@ __device__ __forceinline__ void up_tile_wide_bf16(const MoeArgs &a, int first, i
     const bool active = my_ntf > 0;
 
     const uint32_t row_bytes = (uint32_t)K * 2u;
-    const char *w_gate = a.w1 + ((int64_t)e * N + h0) * K * 2;
+    // this workgroup's share of the contraction (all of it unless the tile is SPLIT)
+    const int n_slabs_all = (int)(row_bytes / ring128::kRB);
+    const int slab0 = SPLIT ? job.part * n_slabs_all / job.parts : 0;
+    const int n_slabs = SPLIT ? (job.part + 1) * n_slabs_all / job.parts - slab0 : n_slabs_all;
+    const char *w_gate = a.w1 + ((int64_t)e * N + h0) * K * 2 + slab0 * ring128::kRB;
     ring128::Loader ld;
-    ld.setup(tid, a.x, w_gate, w_gate + (int64_t)H * K * 2, row_bytes, ntf0, ntf1,
+    ld.setup(tid, a.x + slab0 * ring128::kRB, w_gate, w_gate + (int64_t)H * K * 2, row_bytes, ntf0, ntf1,
              [&](int row) { return (uint32_t)max(ri.tok[row], 0) * row_bytes; });  // dead rows read token 0
 
     const int wrow[2] = {32 * w4, 128 + 32 * w4};
     f32x16 acc[2][4];
     zero_acc(acc);
-    const int n_slabs = (int)(row_bytes / ring128::kRB);
     const int start = slab_rotation128(n_slabs);
     const int tok_region = grp * ring128::kGroupRegion;
     if (active) ring128::main_loop<NTF, true, true>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
     else ring128::main_loop<NTF, true, false>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
+    if constexpr (SPLIT) {
+        if (!join_parts(a, job, acc, reinterpret_cast<int *>(lds + 4 * ring128::kUnitBytes))) return;
+    }
 
     char *tile = lds + grp * (kBlockRows * kActPitchBf16);
     if (active) swiglu_epilogue<DT_BF16, NTF>(acc, tile, nullptr, w4, lane);
@@ -498,22 +560,26 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
     RowInfo<2> &ri = *reinterpret_cast<RowInfo<2> *>(lds + L::kRowInfoOff);
     Job j;
     if (!resolve_job(a, j)) return;
-    const int first = j.first, nb = j.nb, ht = j.wt, e = j.e, n_sub = j.n_sub;
-    const int ntf = load_row_info<2>(a, first, nb, ri);
+    const int ntf = load_row_info<2>(a, j.first, j.nb, ri);
     if (ntf == 0) return;
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {  // one weight tile per workgroup on this path (see launch_pipeline)
-        if (skinny) up_tile_ring<DT, kSkinnyRB, 1, false>(a, first, ht, 1, e, ri, lds, nullptr);
-        else if (ntf == 1) up_tile_wide_bf16<1>(a, first, ht, e, ri, lds);
-        else if (ntf == 2) up_tile_wide_bf16<2>(a, first, ht, e, ri, lds);
-        else up_tile_wide_bf16<4>(a, first, ht, e, ri, lds);
+        j.n_sub = 1;
+        if (skinny) up_tile_ring<DT, kSkinnyRB, 1, false>(a, j, ri, lds, nullptr);
+        else if (j.parts > 1) {  // one of the workgroups that share a tile of the kernel's tail
+            if (ntf == 1) up_tile_wide_bf16<1, true>(a, j, ri, lds);
+            else if (ntf == 2) up_tile_wide_bf16<2, true>(a, j, ri, lds);
+            else up_tile_wide_bf16<4, true>(a, j, ri, lds);
+        } else if (ntf == 1) up_tile_wide_bf16<1, false>(a, j, ri, lds);
+        else if (ntf == 2) up_tile_wide_bf16<2, false>(a, j, ri, lds);
+        else up_tile_wide_bf16<4, false>(a, j, ri, lds);
     } else {
         uint32_t *act_sc_lds = reinterpret_cast<uint32_t *>(lds + L::kActScaleOff);
         const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-        if (ntf == 1) up_tile_ring<DT, kSkinnyRB, 1, false>(a, first, ht, n_sub, e, ri, lds, act_sc_lds);
-        else if (ntf == 2) up_tile_ring<DT, kPartRB, 2, false>(a, first, ht, n_sub, e, ri, lds, act_sc_lds);
-        else if (full) up_tile_ring<DT, 64, 4, true>(a, first, ht, n_sub, e, ri, lds, act_sc_lds);
-        else up_tile_ring<DT, kPartRB, 4, false>(a, first, ht, n_sub, e, ri, lds, act_sc_lds);
+        if (ntf == 1) up_tile_ring<DT, kSkinnyRB, 1, false>(a, j, ri, lds, act_sc_lds);
+        else if (ntf == 2) up_tile_ring<DT, kPartRB, 2, false>(a, j, ri, lds, act_sc_lds);
+        else if (full) up_tile_ring<DT, 64, 4, true>(a, j, ri, lds, act_sc_lds);
+        else up_tile_ring<DT, kPartRB, 4, false>(a, j, ri, lds, act_sc_lds);
     }
 }
 
@@ -681,20 +747,21 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
 // tiles), z = part | parts << 4 | tail slot << 8 (see TailSplit).
 //
 // Workgroups start in the order of their ids, so the last `per_xcd_tail` positions of every XCD's range
-// are the jobs that would run while most CUs have nothing left to do.  The down kernel splits the
+// are the jobs that would run while most CUs have nothing left to do.  The bf16 kernels split the
 // contraction of each of them over `parts` workgroups: part 0 stays in place, the others go behind the
-// list proper (from entry `extra_base` on) and write partial tiles to y_tail, which the finalize
-// kernel adds (tail_tab tells it which tiles have parts and where).
-constexpr int kTailSlots = 192;  // partial tiles y_tail holds (256 x 256 bf16 each)
+// list proper (from entry `extra_base` on).  Down kernel: they write partial tiles to y_tail, which the
+// finalize kernel adds (tail_tab tells it which tiles have parts and where).  Up kernel: see join_parts.
+constexpr int kTailSlots = 192;  // work list entries behind the list proper = partial tiles y_tail holds
 struct TailSplit {
     int parts;         // 1: no split
     int per_xcd_tail;  // jobs split at the end of each XCD's range
     int extra_base;    // first work list entry of the parts > 0
-    int *tail_tab;     // per (block, weight tile): 0, or first slot << 8 | block inside its tile << 4 | parts
+    int *tail_tab;     // down kernel: per (block, weight tile) 0, or first y_tail tile << 8 | block inside its tile << 4 | parts
 };
 
-// How the tail of `n_jobs` down jobs on `n_cus` CUs is split; every part gets at least one slab.
-__device__ __forceinline__ void plan_tail_split(TailSplit &ts, int n_jobs, int n_cus, int n_slabs) {
+// How the tail of `n_jobs` jobs on `n_cus` CUs is split: at most `max_jobs` of them, every part gets at
+// least one slab, and the parts > 0 fit the kTailSlots entries behind the list.
+__device__ __forceinline__ void plan_tail_split(TailSplit &ts, int n_jobs, int n_cus, int n_slabs, int max_jobs) {
     ts.parts = 1;
     ts.per_xcd_tail = 0;
     if (n_cus <= 0 || n_jobs <= 0) return;
@@ -702,6 +769,7 @@ __device__ __forceinline__ void plan_tail_split(TailSplit &ts, int n_jobs, int n
     if (rest == 0 || rounds >= 16) return;  // nothing left over, or too little to matter
     int parts = min(min(4, n_slabs), n_cus / rest);
     const int per_xcd_tail = (rest + 7) >> 3;
+    if (per_xcd_tail * 8 > max_jobs) return;
     while (parts > 1 && per_xcd_tail * 8 * (parts - 1) > kTailSlots) --parts;
     if (parts < 2) return;
     ts.parts = parts;
@@ -721,11 +789,13 @@ __device__ __forceinline__ void emit_work(int4 *work, int n_wt, int per_job, int
         const int x = first | (nb << 28), y = wt | (e << 16) | ((cnt - 1) << 26);
         const int pos = l % per_xcd, xcd = l / per_xcd;
         if (ts != nullptr && ts->parts > 1 && pos >= per_xcd - ts->per_xcd_tail) {
-            const int slot = ((pos - (per_xcd - ts->per_xcd_tail)) * 8 + xcd) * (ts->parts - 1);
+            const int slot = (pos - (per_xcd - ts->per_xcd_tail)) * 8 + xcd;  // number of the tail job
             const int z = (ts->parts << 4) | (slot << 8);
+            const int extra = slot * (ts->parts - 1);
             work[8 * pos + xcd] = make_int4(x, y, z, 0);
-            for (int p = 1; p < ts->parts; ++p) work[ts->extra_base + slot + p - 1] = make_int4(x, y, z | p, 0);
-            for (int b = 0; b < nb; ++b) ts->tail_tab[(first + b) * n_wt + wt] = (slot << 8) | (b << 4) | ts->parts;
+            for (int p = 1; p < ts->parts; ++p) work[ts->extra_base + extra + p - 1] = make_int4(x, y, z | p, 0);
+            if (ts->tail_tab != nullptr)
+                for (int b = 0; b < nb; ++b) ts->tail_tab[(first + b) * n_wt + wt] = (extra << 8) | (b << 4) | ts->parts;
         } else {
             work[8 * pos + xcd] = make_int4(x, y, 1 << 4, 0);
         }
@@ -741,8 +811,8 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
                                                            int n_blocks, int2 *tiles, int *n_tiles,
                                                            int4 *work_up, int n_wt_up, int per_job_up, int grid_up,
                                                            int4 *work_down, int n_wt_down, int per_job_down,
-                                                           int grid_down, int split_cus, int down_slabs,
-                                                           int *tail_tab, int num_experts,
+                                                           int grid_down, int split_cus, int up_slabs, int down_slabs,
+                                                           int *tail_tab, int *up_counters, int num_experts,
                                                            const int32_t *sorted_ids, int sorted_num, int32_t *inv,
                                                            int n_pairs, int do_invert, const uint8_t *x_scales,
                                                            uint32_t *xs_tiled, int nkt, int top_k, int M) {
@@ -753,6 +823,7 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
         for (int i = tid; i < grid_down; i += 256) work_down[i] = make_int4(-1, -1, 0, 0);
         if (tail_tab != nullptr)
             for (int i = tid; i < n_blocks * n_wt_down; i += 256) tail_tab[i] = 0;
+        if (up_counters != nullptr && tid < kUpTailJobs) up_counters[tid] = 0;
         const int n_live = min((ntpp[0] + kBlockRows - 1) / kBlockRows, n_blocks);
         if (tid == 0) { s_carry[0] = 0; s_carry[1] = 0; }
         __syncthreads();
@@ -793,16 +864,21 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
         if (tid == 0) n_tiles[0] = nt;
         __threadfence_block();
         __syncthreads();  // tiles written above are read below by other threads
-        TailSplit ts;
+        // contraction splits of the two kernels' tails (bf16 only: tail_tab and up_counters are null else)
+        TailSplit ts, ts_up;
         ts.extra_base = grid_down - kTailSlots;
         ts.tail_tab = tail_tab;
         plan_tail_split(ts, tail_tab != nullptr ? nt * ((n_wt_down + per_job_down - 1) / per_job_down) : 0, split_cus,
-                        down_slabs);
+                        down_slabs, kTailSlots);
+        ts_up.extra_base = grid_up - kTailSlots;
+        ts_up.tail_tab = nullptr;
+        plan_tail_split(ts_up, up_counters != nullptr ? nt * ((n_wt_up + per_job_up - 1) / per_job_up) : 0, split_cus,
+                        up_slabs, kUpTailJobs);
         for (int t = tid; t < nt; t += 256) {
             const int2 tl = tiles[t];
             const int e = expert_ids[tl.x];
             if (e < 0 || e >= num_experts) continue;  // nothing to compute for a block without an expert
-            emit_work(work_up, n_wt_up, per_job_up, t, nt, tl.x, tl.y, e, nullptr);
+            emit_work(work_up, n_wt_up, per_job_up, t, nt, tl.x, tl.y, e, &ts_up);
             emit_work(work_down, n_wt_down, per_job_down, t, nt, tl.x, tl.y, e, &ts);
         }
     }
@@ -910,7 +986,8 @@ __global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int3
 // ------------------------------------------------------------------------------------------ host
 
 struct WorkspaceLayout {
-    size_t n_tiles_off, tiles_off, work_up_off, work_down_off, tail_tab_off, y_tail_off, inv_off, y_off, act_off,
+    size_t n_tiles_off, up_counters_off, tiles_off, work_up_off, work_down_off, tail_tab_off, y_tail_off,
+        up_partials_off, inv_off, y_off, act_off,
         act_scales_off, xs_tiled_off, total;
 };
 
@@ -922,10 +999,12 @@ static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_
     size_t off = 0;
     l.n_tiles_off = off;
     off += 256;
+    l.up_counters_off = off;
+    off += kUpTailJobs * sizeof(int32_t);
     l.tiles_off = off;
     off = align_up(off + blocks * sizeof(int2), 256);
     l.work_up_off = off;
-    off = align_up(off + align_up(blocks * (H / 128), 8) * sizeof(int4), 256);
+    off = align_up(off + (align_up(blocks * (H / 128), 8) + kTailSlots) * sizeof(int4), 256);
     l.work_down_off = off;
     const size_t n_wt_down = ((size_t)K + kWRows - 1) / kWRows;
     off = align_up(off + (align_up(blocks * n_wt_down, 8) + kTailSlots) * sizeof(int4), 256);
@@ -933,6 +1012,8 @@ static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_
     if (dt == DT_BF16) off = align_up(off + blocks * n_wt_down * sizeof(int32_t), 256);
     l.y_tail_off = off;
     if (dt == DT_BF16) off = align_up(off + (size_t)kTailSlots * kWRows * kWRows * 2, 256);
+    l.up_partials_off = off;  // 4 parts x 512 threads x 128 floats per job
+    if (dt == DT_BF16) off = align_up(off + (size_t)kUpTailJobs * 4 * 512 * 128 * sizeof(float), 256);
     l.inv_off = off;
     off = align_up(off + (size_t)M * (size_t)std::max(top_k, 1) * sizeof(int32_t), 256);
     l.y_off = off;
@@ -988,7 +1069,8 @@ struct SchedBuffers {
     int *n_tiles;
     int4 *work_up;
     int4 *work_down;
-    int *tail_tab;  // null: the down kernel's tail is not split (mxfp8)
+    int *tail_tab;     // null: the down kernel's tail is not split (mxfp8)
+    int *up_counters;  // null: the up kernel's tail is not split (mxfp8)
 };
 
 template <int DT>
@@ -1002,8 +1084,8 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
     const int n_wt_down = (a.K + kWRows - 1) / kWRows;
     const int per_up = tiles_per_workgroup(DT, false, a.n_blocks, a.n_wtiles);
     const int per_down = tiles_per_workgroup(DT, true, a.n_blocks, n_wt_down);
-    const int grid_up = grid_for(a.n_blocks * ((a.n_wtiles + per_up - 1) / per_up));
-    // the parts > 0 of split tail jobs sit behind the list proper
+    const int grid_up = grid_for(a.n_blocks * ((a.n_wtiles + per_up - 1) / per_up)) + kTailSlots;
+    // (the parts > 0 of split tail jobs sit behind the lists proper)
     const int grid_down = grid_for(a.n_blocks * ((n_wt_down + per_down - 1) / per_down)) + kTailSlots;
     {
         // the work lists are needed by the two kernels even when the rest of the prologue is masked off
@@ -1011,7 +1093,8 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
         const int blocks = do_invert ? std::max(1, std::min((a.sorted_num + 255) / 256, 1024)) : 1;
         hipLaunchKernelGGL(moe_prologue_kernel, dim3(blocks), dim3(256), 0, s, a.expert_ids, a.ntpp, a.n_blocks,
                            sb.tiles, sb.n_tiles, sb.work_up, a.n_wtiles, per_up, grid_up,
-                           sb.work_down, n_wt_down, per_down, grid_down, resident_grid(), a.H * 2 / 128, sb.tail_tab, a.E,
+                           sb.work_down, n_wt_down, per_down, grid_down, resident_grid(), a.K * 2 / 128, a.H * 2 / 128,
+                           sb.tail_tab, sb.up_counters, a.E,
                            a.sorted_ids, a.sorted_num, a.inv, a.M * a.top_k, do_invert, a.x_scales, a.xs_tiled,
                            a.K >> 7, a.top_k, a.M);
     }
@@ -1047,6 +1130,7 @@ static SchedBuffers sched_buffers(char *ws, const WorkspaceLayout &l) {
     sb.work_up = reinterpret_cast<int4 *>(ws + l.work_up_off);
     sb.work_down = reinterpret_cast<int4 *>(ws + l.work_down_off);
     sb.tail_tab = l.y_tail_off > l.tail_tab_off ? reinterpret_cast<int *>(ws + l.tail_tab_off) : nullptr;
+    sb.up_counters = sb.tail_tab != nullptr ? reinterpret_cast<int *>(ws + l.up_counters_off) : nullptr;
     return sb;
 }
 
@@ -1110,6 +1194,8 @@ extern "C" int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2,
     char *ws = static_cast<char *>(workspace);
     a.y = ws + l.y_off;
     a.y_tail = ws + l.y_tail_off;
+    a.up_partials = reinterpret_cast<float *>(ws + l.up_partials_off);
+    a.up_counters = reinterpret_cast<int *>(ws + l.up_counters_off);
     a.inv = reinterpret_cast<int32_t *>(ws + l.inv_off);
     a.act = ws + l.act_off;
     a.top_k = top_k; a.M = M; a.K = K; a.N = N; a.H = N / 2; a.E = num_experts; a.sorted_num = sorted_num;

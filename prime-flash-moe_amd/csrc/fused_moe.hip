@@ -6,15 +6,17 @@
 //
 // Pipeline of one call (all on the caller's stream):
 //   prologue (pair blocks into row tiles, build the two work lists, invert the sorted order:
-//             pair id -> sorted row)
+//             pair id -> sorted row; mxfp8: re-tile the scales of the gathered x rows)
 //   -> up kernel (gate/up GEMM + SwiGLU, activation tile -> workspace)
 //   -> down kernel (y[sorted row, :K] = act . W2[e]^T, bf16, -> workspace)
 //   -> finalize: out[t] = bf16(sum over the token's pairs p of w[p] * y[row(p)]), fp32 sum in pair
 //      order; split == 0: added to `out` (the reference's accumulate-into-out contract of its
 //      single-kernel path), split != 0: `out` overwritten.
 // Both values of `split` run the same kernels: on this hardware the two-kernel pipeline is the faster
-// one at every shape, so `split` only selects what finalize does with `out`.  No atomics: the result
-// is a pure function of the inputs.
+// one at every shape, so `split` only selects what finalize does with `out`.  The jobs of a bf16 kernel
+// that start last share their tile's contraction among several workgroups (see TailSplit).  No value
+// is accumulated with atomics and every sum has a fixed order: the result is a pure function of the
+// inputs.
 #include <algorithm>
 
 #include "moe_ring.h"
@@ -35,7 +37,7 @@ struct MoeArgs {
     const int32_t *expert_ids;
     const int32_t *ntpp;
     const float *topk_w;
-    char *act;            // (sorted_num, H) activation workspace (split pipeline)
+    char *act;            // (sorted_num, H) activation workspace, bf16 or e4m3
     // e8m0 scales of the token-side operands of the two mxfp8 GEMMs, as the loaders want them: one
     // dword (4 scales = 128 contraction elements) per row, [sorted block][128-wide K tile][row in block],
     // so that the 64 lanes of a copy instruction read 256 contiguous bytes.
@@ -583,8 +585,9 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
     }
 }
 
-// Down kernel of the split pipeline: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T,
-// full reduction over H inside the workgroup (no split-K), then w[row] * y added to accum[token].
+// Down kernel tile on the stage ring: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T, the
+// whole reduction over H inside the workgroup unless the job is one part of a split tail tile; the
+// routing weights are applied later, by finalize_kernel.
 template <int DT, int RB, int NTF, bool FULL>
 __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, const Job &job, RowInfo<2> &ri, char *lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;

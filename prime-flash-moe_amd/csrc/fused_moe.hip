@@ -1181,6 +1181,8 @@ extern "C" int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2,
     PMOE_REQUIRE(!split || stages <= 4, "split=True requires stages<=4, got stages=%d", stages);
     PMOE_REQUIRE(top_k > 0 && num_experts > 0 && sorted_num >= 0, "fused_moe_bf16: bad top_k / num_experts / sorted_num");
     PMOE_REQUIRE(num_experts <= 1024, "fused_moe_bf16: at most 1024 experts, got %d", num_experts);
+    // the gather addresses a token row by a 32-bit byte offset from x
+    PMOE_REQUIRE((uint64_t)M * (uint64_t)K * 2u < (1ull << 32), "fused_moe_bf16: x must be smaller than 4 GiB, got %d x %d", M, K);
     PMOE_REQUIRE(x && w && w2 && out && sorted_token_ids && expert_idxs && num_tokens_post_padded && topk_weights,
                  "fused_moe_bf16: null pointer");
     const WorkspaceLayout l = workspace_layout(DT_BF16, M, K, N, sorted_num, top_k);
@@ -1220,6 +1222,8 @@ extern "C" int pmoe_fused_moe_mxfp8(const void *x, const void *x_scales, const v
     PMOE_REQUIRE(bpc == 1, "mxfp8 supports bpc=1 only");
     PMOE_REQUIRE(top_k > 0 && num_experts > 0 && sorted_num >= 0, "fused_moe_mxfp8: bad top_k / num_experts / sorted_num");
     PMOE_REQUIRE(num_experts <= 1024, "fused_moe_mxfp8: at most 1024 experts, got %d", num_experts);
+    // the gather addresses a token row by a 32-bit byte offset from x
+    PMOE_REQUIRE((uint64_t)M * (uint64_t)K < (1ull << 32), "fused_moe_mxfp8: x must be smaller than 4 GiB, got %d x %d", M, K);
     PMOE_REQUIRE(x && x_scales && w && w_scales && w2 && w2_scales && out && sorted_token_ids && expert_idxs &&
                      num_tokens_post_padded && topk_weights,
                  "fused_moe_mxfp8: null pointer");

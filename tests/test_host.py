@@ -53,6 +53,15 @@ def test_workspace_query_and_c_side_validation_need_no_gpu():
     assert rc == 1 and b"multiple of 256" in lib.pmoe_last_error()
     with pytest.raises(RuntimeError, match="multiple of 256"):
         _native.check(rc)
+    # limits of the kernels' own encodings: expert number in 10 bits, 32-bit byte offsets into x
+    rc = lib.pmoe_fused_moe_bf16(None, None, None, None, None, None, None, None, 2, 16, 4096, 512, 2000, 2048,
+                                 128, 64, 4, 2, 1, 1, 1, None, 0, None)
+    assert rc == 1 and b"at most 1024 experts" in lib.pmoe_last_error()
+    rc = lib.pmoe_fused_moe_bf16(None, None, None, None, None, None, None, None, 2, 1 << 20, 4096, 512, 8, 2048,
+                                 128, 64, 4, 2, 1, 1, 1, None, 0, None)
+    assert rc == 1 and b"smaller than 4 GiB" in lib.pmoe_last_error()
+    rc = lib.pmoe_fused_moe_mxfp8(*([None] * 11), 2, 1 << 20, 4096, 512, 8, 2048, 128, 64, 4, 2, 1, 1, None, 0, None)
+    assert rc == 1 and b"smaller than 4 GiB" in lib.pmoe_last_error()
 
 
 def test_missing_library_fails_loudly(monkeypatch):

@@ -76,7 +76,10 @@ size_t pmoe_fused_moe_mxfp8_workspace_bytes(int M, int K, int N, int num_experts
  * workspace; `split` selects only how the last kernel treats `out`.
  * block_n / warp_n / stages are validated exactly as the reference does and then
  * ignored (they size Blackwell thread blocks and smem rings); block_m must be 128,
- * bpc == cpc == 1, K % 128 == 0, N % 256 == 0.
+ * bpc == cpc == 1, K % 128 == 0, N % 256 == 0.  Limits of this implementation, checked:
+ * num_experts <= 1024 (as moe_align) and x smaller than 4 GiB.
+ * The workspace is scratch of this one call: calls that may run at the same time need
+ * their own.
  */
 int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2, void *out,
                         const int32_t *sorted_token_ids, const int32_t *expert_idxs,
@@ -92,7 +95,8 @@ int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2, void *out,
  *   128x4 blocked tiles [E][N/128][K/128][512]; w2 (E,K,N/2) e4m3 + w2_scales blocked
  *   [E][K/128][(N/2)/128][512].  The SwiGLU activation is requantised on chip to e4m3
  *   with one e8m0 scale per 32 elements along N/2 before the down projection.
- *   K % 256 == 0, N % 256 == 0, bpc == 1, block_m == 128.
+ *   K % 256 == 0, N % 256 == 0, bpc == 1, block_m == 128; num_experts <= 1024 and x
+ *   smaller than 4 GiB as for fused_moe_bf16.
  */
 int pmoe_fused_moe_mxfp8(const void *x, const void *x_scales, const void *w, const void *w_scales,
                          const void *w2, const void *w2_scales, void *out,

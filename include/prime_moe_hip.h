@@ -53,6 +53,19 @@ int pmoe_moe_align(const int32_t *topk_ids, int32_t *sorted_token_ids, int32_t *
                    int pad_to, int max_padded, int max_blocks, void *stream);
 
 /*
+ * The same sort with scratch memory from the caller, which lets it spread over many
+ * workgroups (three launches) when n is large; no counterpart in the reference, whose
+ * kernel is one thread block for any n.  The query returns 0 for sizes the single
+ * workgroup of pmoe_moe_align handles (then `workspace` may be null); with a null or too
+ * small workspace the call falls back to that single workgroup.  Same output, bit for bit.
+ */
+size_t pmoe_moe_align_workspace_bytes(int n, int num_experts);
+int pmoe_moe_align_ws(const int32_t *topk_ids, int32_t *sorted_token_ids, int32_t *expert_ids,
+                      int32_t *num_tokens_post_padded, int n, int num_experts, int block_m,
+                      int pad_to, int max_padded, int max_blocks, void *workspace,
+                      size_t workspace_bytes, void *stream);
+
+/*
  * Workspace (bytes) the fused calls below need for a problem of this size.  The
  * caller allocates it on the device (any 256-byte aligned buffer) and passes it in.
  * The size does not depend on `split` (both values run the same kernels); the argument

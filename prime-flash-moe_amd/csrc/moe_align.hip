@@ -121,12 +121,196 @@ __global__ __launch_bounds__(NW * 64) void moe_align_kernel(
     }
 }
 
+// ---- many ids: the same sort spread over workgroups, three launches.
+//   count:   workgroup g histograms ids [g S, (g+1) S) -> counts[g][e]
+//   scan:    one workgroup turns counts[.][e] into exclusive bases over the workgroups, writes the
+//            per-expert totals cnt[e], the padded exclusive prefix offs[0..E], the total and expert_ids
+//   scatter: workgroup g sorts its slice as the single-workgroup kernel does (per-wave histogram,
+//            ballot ranks) and writes pair id i to offs[e] + counts[g][e] + base of its wave + rank;
+//            it also writes -1 to the padding slots of its share of the output (a slot is padding if
+//            it lies at or behind cnt[e] inside its expert's padded range, or behind the total), so
+//            no slot is written twice and no order between workgroups is needed.
+// Slices are contiguous and ascending in g, waves inside a slice likewise: the order inside an expert is
+// ascending pair id, bit for bit what the single workgroup produces.
+constexpr int kSliceIds = 8192;       // ids per workgroup
+constexpr int kSingleMaxIds = 16384;  // up to here one workgroup is faster than three launches
+
+struct AlignScratch {
+    int32_t *counts;  // [G][E]
+    int32_t *offs;    // [E + 1]
+    int32_t *cnt;     // [E]
+};
+
+__global__ __launch_bounds__(1024) void align_count_kernel(const int32_t *__restrict__ topk_ids, int n, int E,
+                                                           int32_t *__restrict__ counts) {
+    extern __shared__ int32_t smem[];
+    const int tid = threadIdx.x, g = blockIdx.x;
+    for (int e = tid; e < E; e += 1024) smem[e] = 0;
+    __syncthreads();
+    const int beg = g * kSliceIds, end = min(n, beg + kSliceIds);
+    for (int i = beg + tid; i < end; i += 1024) {
+        const int e = topk_ids[i];
+        if (e >= 0 && e < E) atomicAdd(smem + e, 1);
+    }
+    __syncthreads();
+    for (int e = tid; e < E; e += 1024) counts[g * E + e] = smem[e];
+}
+
+__global__ __launch_bounds__(1024) void align_scan_kernel(AlignScratch sc, int G, int E, int block_m, int pad_to,
+                                                          int max_blocks, int32_t *__restrict__ expert_ids,
+                                                          int32_t *__restrict__ num_tokens_post_padded) {
+    extern __shared__ int32_t smem[];
+    int32_t *offs = smem;            // [E + 1]
+    int32_t *padc = smem + (E + 1);  // [E]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int e = tid; e < E; e += 1024) {
+        int run = 0;
+        for (int g = 0; g < G; ++g) {
+            const int c = sc.counts[g * E + e];
+            sc.counts[g * E + e] = run;
+            run += c;
+        }
+        sc.cnt[e] = run;
+        padc[e] = (run + pad_to - 1) / pad_to * pad_to;
+    }
+    __syncthreads();
+    if (wave == 0) {  // exclusive prefix over experts, as in the single-workgroup kernel
+        const int chunk = (E + 63) >> 6;
+        const int b = lane * chunk;
+        int local = 0;
+        for (int j = 0; j < chunk; ++j)
+            if (b + j < E) local += padc[b + j];
+        int incl = local;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            int v = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += v;
+        }
+        int run = incl - local;
+        for (int j = 0; j < chunk; ++j)
+            if (b + j < E) {
+                offs[b + j] = run;
+                run += padc[b + j];
+            }
+        if (lane == 63) offs[E] = incl;
+    }
+    __syncthreads();
+    const int total = offs[E];
+    if (tid == 0) num_tokens_post_padded[0] = total;
+    for (int e = tid; e <= E; e += 1024) sc.offs[e] = offs[e];
+    for (int j = tid; j < max_blocks; j += 1024) {
+        const int row = j * block_m;
+        int owner = E - 1;
+        if (row < total) {
+            int lo = 0, hi = E - 1;
+            while (lo < hi) {
+                int mid = (lo + hi + 1) >> 1;
+                if (offs[mid] <= row) lo = mid;
+                else hi = mid - 1;
+            }
+            owner = lo;
+        }
+        expert_ids[j] = owner;
+    }
+}
+
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void align_scatter_kernel(const int32_t *__restrict__ topk_ids,
+                                                                int32_t *__restrict__ sorted_token_ids,
+                                                                AlignScratch sc, int n, int E, int max_padded,
+                                                                int id_bits) {
+    extern __shared__ int32_t smem[];
+    int32_t *offs = smem;                  // [E + 1]
+    int32_t *cnt = smem + (E + 1);         // [E]
+    int32_t *wbase = smem + (2 * E + 1);   // [NW][E] per-wave counts, then running bases
+    constexpr int NT = NW * 64;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = blockIdx.x, G = gridDim.x;
+    for (int e = tid; e <= E; e += NT) offs[e] = sc.offs[e];
+    for (int e = tid; e < E; e += NT) cnt[e] = sc.cnt[e];
+    for (int i = tid; i < NW * E; i += NT) wbase[i] = 0;
+    __syncthreads();
+
+    // this workgroup's share of the -1 fill
+    {
+        const int total = offs[E];
+        const int per = (max_padded + G - 1) / G;
+        const int pend = min(max_padded, (g + 1) * per);
+        for (int pos = g * per + tid; pos < pend; pos += NT) {
+            bool pad = pos >= total;
+            if (!pad) {
+                int lo = 0, hi = E - 1;
+                while (lo < hi) {
+                    int mid = (lo + hi + 1) >> 1;
+                    if (offs[mid] <= pos) lo = mid;
+                    else hi = mid - 1;
+                }
+                pad = pos - offs[lo] >= cnt[lo];
+            }
+            if (pad) sorted_token_ids[pos] = -1;
+        }
+    }
+
+    // the slice, one contiguous run of a multiple of 64 ids per wave
+    const int sbeg = g * kSliceIds, send = min(n, sbeg + kSliceIds);
+    constexpr int per_wave = kSliceIds / NW;
+    const int beg = sbeg + wave * per_wave;
+    const int end = min(send, beg + per_wave);
+    int32_t *mine = wbase + wave * E;
+    for (int i = beg + lane; i < end; i += 64) {
+        const int e = topk_ids[i];
+        if (e >= 0 && e < E) atomicAdd(mine + e, 1);
+    }
+    __syncthreads();
+    for (int e = tid; e < E; e += NT) {
+        int run = offs[e] + sc.counts[g * E + e];  // first slot of this workgroup's ids of expert e
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            const int c = wbase[w * E + e];
+            wbase[w * E + e] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    for (int i0 = beg; i0 < end; i0 += 64) {
+        const int i = i0 + lane;
+        const int e = (i < end) ? topk_ids[i] : -1;
+        const bool valid = e >= 0 && e < E;
+        unsigned long long peers = __ballot(valid);
+        for (int b = 0; b < id_bits; ++b) {
+            const bool bit = (e >> b) & 1;
+            const unsigned long long set = __ballot(bit);
+            peers &= bit ? set : ~set;
+        }
+        if (valid) {
+            const int rank = __popcll(peers & ((1ull << lane) - 1ull));
+            const int c = __popcll(peers);
+            const int base = mine[e];
+            sorted_token_ids[base + rank] = i;
+            if (rank == c - 1) mine[e] = base + c;  // one writer per group, after all reads
+        }
+    }
+}
+
 }  // namespace
+
+extern "C" size_t pmoe_moe_align_workspace_bytes(int n, int num_experts) {
+    if (n <= kSingleMaxIds || num_experts <= 0 || num_experts > kMaxExperts) return 0;
+    const size_t G = ((size_t)n + kSliceIds - 1) / kSliceIds;
+    return sizeof(int32_t) * (G * (size_t)num_experts + 2 * (size_t)num_experts + 1);
+}
 
 extern "C" int pmoe_moe_align(const int32_t *topk_ids, int32_t *sorted_token_ids,
                               int32_t *expert_ids, int32_t *num_tokens_post_padded, int n,
                               int num_experts, int block_m, int pad_to, int max_padded,
                               int max_blocks, void *stream) {
+    return pmoe_moe_align_ws(topk_ids, sorted_token_ids, expert_ids, num_tokens_post_padded, n, num_experts, block_m,
+                             pad_to, max_padded, max_blocks, nullptr, 0, stream);
+}
+
+extern "C" int pmoe_moe_align_ws(const int32_t *topk_ids, int32_t *sorted_token_ids, int32_t *expert_ids,
+                                 int32_t *num_tokens_post_padded, int n, int num_experts, int block_m, int pad_to,
+                                 int max_padded, int max_blocks, void *workspace, size_t workspace_bytes,
+                                 void *stream) {
     PMOE_REQUIRE(num_experts > 0 && block_m > 0 && pad_to > 0, "moe_align: block_m, bpc and num_experts must be positive");
     PMOE_REQUIRE(num_experts <= kMaxExperts, "moe_align supports at most 1024 experts, got %d", num_experts);
     PMOE_REQUIRE(n >= 0 && max_padded >= 0 && max_blocks >= 0, "moe_align: negative size");
@@ -140,6 +324,31 @@ extern "C" int pmoe_moe_align(const int32_t *topk_ids, int32_t *sorted_token_ids
     int id_bits = 1;
     while ((1 << id_bits) < num_experts) ++id_bits;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t ws_need = pmoe_moe_align_workspace_bytes(n, num_experts);
+    if (ws_need > 0 && workspace != nullptr && workspace_bytes >= ws_need) {
+        PMOE_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 3) == 0, "moe_align: workspace must be 4-byte aligned");
+        const int G = (n + kSliceIds - 1) / kSliceIds;
+        AlignScratch sc;
+        sc.counts = static_cast<int32_t *>(workspace);
+        sc.offs = sc.counts + (size_t)G * num_experts;
+        sc.cnt = sc.offs + num_experts + 1;
+        hipLaunchKernelGGL(align_count_kernel, dim3(G), dim3(1024), sizeof(int32_t) * num_experts, s, topk_ids, n,
+                           num_experts, sc.counts);
+        hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(1024), sizeof(int32_t) * (2 * num_experts + 1), s, sc, G,
+                           num_experts, block_m, pad_to, max_blocks, expert_ids, num_tokens_post_padded);
+        if (num_experts <= 512) {
+            constexpr int NW = 16;
+            hipLaunchKernelGGL(align_scatter_kernel<NW>, dim3(G), dim3(NW * 64),
+                               sizeof(int32_t) * (size_t)(2 * num_experts + 1 + NW * num_experts), s, topk_ids,
+                               sorted_token_ids, sc, n, num_experts, max_padded, id_bits);
+        } else {
+            constexpr int NW = 8;
+            hipLaunchKernelGGL(align_scatter_kernel<NW>, dim3(G), dim3(NW * 64),
+                               sizeof(int32_t) * (size_t)(2 * num_experts + 1 + NW * num_experts), s, topk_ids,
+                               sorted_token_ids, sc, n, num_experts, max_padded, id_bits);
+        }
+        return pmoe::check_launch("moe_align launch");
+    }
     if (num_experts <= 512) {
         constexpr int NW = 16;
         size_t smem = sizeof(int32_t) * (size_t)(2 * num_experts + 1 + NW * num_experts);

@@ -74,11 +74,14 @@ def _moe_align_impl(topk_ids, num_experts, block_m, bpc):
     expert_ids = torch.empty((max_blocks,), dtype=torch.int32, device=dev)
     num_tokens_post_padded = torch.empty((1,), dtype=torch.int32, device=dev)
     lib = _native.load()
+    # many ids: scratch for the multi-workgroup sort (0 bytes when one workgroup does it)
+    ws_bytes = lib.pmoe_moe_align_workspace_bytes(n, num_experts)
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes else None
     with torch.cuda.device(dev):
-        _native.check(lib.pmoe_moe_align(
+        _native.check(lib.pmoe_moe_align_ws(
             topk_ids.data_ptr(), sorted_token_ids.data_ptr(), expert_ids.data_ptr(),
             num_tokens_post_padded.data_ptr(), n, num_experts, block_m, pad_to, max_padded,
-            max_blocks, _stream_ptr(dev)))
+            max_blocks, ws.data_ptr() if ws is not None else None, ws_bytes, _stream_ptr(dev)))
     return sorted_token_ids, expert_ids, num_tokens_post_padded
 
 

@@ -67,3 +67,54 @@ def test_align_errors(device):
         torch.ops.prime_moe.moe_align(ids, 4, 0, 1)
     with pytest.raises(RuntimeError):
         torch.ops.prime_moe.moe_align(torch.zeros((8, 2), device=device, dtype=torch.int32)[:, 0], 4, 128, 1)
+
+
+@pytest.mark.parametrize("T,top_k,E", [
+    (16385, 1, 8),        # one id past what a single workgroup takes: three slices, the last with one id
+    (8192, 4, 37),        # whole slices only
+    (20000, 3, 257),      # a hot last expert, odd sizes
+    (30011, 2, 1024),     # the largest expert count, 8 waves per workgroup
+    (40000, 1, 1),        # one expert
+])
+def test_many_ids_spread_over_workgroups(T, top_k, E, device):
+    # above 16384 ids the op sorts with three launches over many workgroups; the result is the
+    # single-workgroup one bit for bit (ascending pair ids inside an expert)
+    rng = np.random.default_rng(T + E)
+    ids = rng.integers(0, E, size=(T, top_k))
+    if E == 257:
+        ids[:, -1] = E - 1
+    _run(ids, E, 128, 1, device)
+
+
+def test_many_ids_with_ids_out_of_range_and_scratch_fallback(device):
+    import prime_moe
+    from prime_moe import _native
+    rng = np.random.default_rng(3)
+    ids = rng.integers(-2, 12, size=50000).astype(np.int32)
+    # ids outside [0, E) are skipped: the expected result is the oracle's on the ids in range, with
+    # its pair numbers mapped back and the arrays extended to the sizes of the full input
+    keep = np.flatnonzero((ids >= 0) & (ids < 8))
+    s_c, e_c, t_c = O.moe_align_fast(ids[keep], 8, 128, 1)
+    _, max_padded, max_blocks = O.moe_align_sizes(50000, 8, 128, 1)
+    s_w = np.full(max_padded, -1, dtype=np.int32)
+    s_w[: s_c.size] = np.where(s_c >= 0, keep[np.maximum(s_c, 0)], -1)
+    e_w = np.full(max_blocks, 7, dtype=np.int32)
+    e_w[: e_c.size] = e_c
+    want = (s_w, e_w, t_c)
+    dev_ids = torch.from_numpy(ids).to(device)
+    got = torch.ops.prime_moe.moe_align(dev_ids, 8, 128, 1)
+    for a, b in zip(got, want):
+        assert np.array_equal(a.cpu().numpy(), b)
+    # the plain entry point (no scratch) sorts the same ids with its single workgroup
+    lib = _native.load()
+    assert lib.pmoe_moe_align_workspace_bytes(50000, 8) == 4 * (7 * 8 + 2 * 8 + 1)
+    assert lib.pmoe_moe_align_workspace_bytes(16384, 8) == 0
+    pad_to, max_padded, max_blocks = prime_moe.align_sizes(50000, 8, 128, 1)
+    s = torch.empty((max_padded,), dtype=torch.int32, device=device)
+    e = torch.empty((max_blocks,), dtype=torch.int32, device=device)
+    t = torch.empty((1,), dtype=torch.int32, device=device)
+    _native.check(lib.pmoe_moe_align(dev_ids.data_ptr(), s.data_ptr(), e.data_ptr(), t.data_ptr(), 50000, 8, 128,
+                                     pad_to, max_padded, max_blocks, torch.cuda.current_stream(device).cuda_stream))
+    torch.cuda.synchronize()
+    for a, b in zip((s, e, t), want):
+        assert np.array_equal(a.cpu().numpy(), b)

@@ -241,21 +241,7 @@ __device__ __forceinline__ void mma_fp8_step(f32x16 (&acc)[2][4], const char *to
         }
 }
 
-// K loop.  COMPUTE = false is the loop of the waves without matrix work (a group without live
-// rows): they only issue their share of the copies and join the barriers.  `tok_region` = byte
-// offset of this wave's group inside a stage's token rows.
-//
-// The slabs are visited in rotated order, starting at slab `start` (even for RB = 64): workgroups
-// that run side by side and share rows then ask for different cache lines at any one time instead
-// of queueing on the same ones.  The sum over K does not depend on the order.
-//
-// FULL (RB = 64 only): the tile has two completely live blocks, so geometry and wait counts are
-// compile-time constants (`lay` must be that geometry); otherwise both are wave-uniform run-time
-// values and the wait count goes through a switch.
-//
-// Slab 0 goes to stage `stage0`, the following ones to the stages behind it (wrapping).  `n_pre`: the
-// caller has already issued slabs 0 .. n_pre - 1 (see pre_issue; a workgroup that runs one tile
-// after another issues them under the previous tile's epilogue).
+// Geometry of the ring in use: the constants of a full tile or the run-time layout.
 template <int DT, int RB, bool FULL>
 __device__ __forceinline__ int stage_bytes(const Layout &lay) {
     return FULL ? FullCfg<DT>::kStageBytes : lay.stage_bytes;
@@ -279,6 +265,21 @@ __device__ __forceinline__ void pre_issue(const Loader<RB> &ld, const Layout &la
         ld.issue(lds + st * SB, slab);
     }
 }
+// K loop.  COMPUTE = false is the loop of the waves without matrix work (a group without live
+// rows): they only issue their share of the copies and join the barriers.  `tok_region` = byte
+// offset of this wave's group inside a stage's token rows.
+//
+// The slabs are visited in rotated order, starting at slab `start` (even for RB = 64): workgroups
+// that run side by side and share rows then ask for different cache lines at any one time instead
+// of queueing on the same ones.  The sum over K does not depend on the order.
+//
+// FULL (RB = 64 only): the tile has two completely live blocks, so geometry and wait counts are
+// compile-time constants (`lay` must be that geometry); otherwise both are wave-uniform run-time
+// values and the wait count goes through a switch.
+//
+// Slab 0 goes to stage `stage0`, the following ones to the stages behind it (wrapping).  `n_pre`: the
+// caller has already issued slabs 0 .. n_pre - 1 (see pre_issue; a workgroup that runs one tile
+// after another issues them under the previous tile's epilogue).
 template <int DT, int RB, int NTF, bool TRANSPOSED, bool COMPUTE, bool FULL>
 __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader<RB> &ld, const Layout &lay, char *lds,
                                           int n_slabs, const int (&wrow)[2], int lane, int tok_region, int start,

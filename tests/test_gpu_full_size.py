@@ -72,7 +72,7 @@ def test_full_size_config(name, n_sample, device):
         c, l2 = cosine(got_s, ref), rel_l2(got_s, ref)
         assert c >= MX_COS_GATE and l2 <= MX_RELL2_GATE, f"{name}: cosine {c}, rel-L2 {l2}"
 
-    # (b) linear in the routing weights (exact up to the order of the fp32 atomics and bf16 rounding)
+    # (b) linear in the routing weights (up to the bf16 rounding of `out`)
     out2 = torch.empty_like(out)
     _run(cfg, inp, sched, out2, True, weights=inp["topk_weights"] * 2.0)
     scale = float(got.abs().max())

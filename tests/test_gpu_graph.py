@@ -24,10 +24,13 @@ def _eager(kind, a, ids, wts, E, top_k):
     return out
 
 
-@pytest.mark.parametrize("kind", ["bf16", "mxfp8"])
-def test_capture_and_replay(kind, device):
+@pytest.mark.parametrize("kind,T,top_k", [
+    ("bf16", 192, 2), ("mxfp8", 192, 2),
+    ("bf16", 4500, 4),  # 18000 ids: the multi-workgroup moe_align and whole rounds of tiles with a split tail
+])
+def test_capture_and_replay(kind, T, top_k, device):
     import prime_moe
-    T, K, E, N, top_k = 192, 512, 8, 512, 2
+    K, E, N = 512, 8, 512
     g = torch.Generator(device=device).manual_seed(3)
     w1 = (torch.randn((E, N, K), device=device, generator=g) / math.sqrt(K)).to(torch.bfloat16)
     w2 = (torch.randn((E, K, N // 2), device=device, generator=g) / math.sqrt(N // 2)).to(torch.bfloat16)

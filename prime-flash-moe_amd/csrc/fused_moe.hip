@@ -295,21 +295,26 @@ __device__ __forceinline__ void store_act_tile(const MoeArgs &a, const char *til
 }
 
 // Contraction split of an up tile: every part stores its accumulators (32 float4 per thread, thread
-// index fastest), makes them visible to the device and counts itself in; the part that counts last
-// adds all parts in part order (its own too, from memory: the same bits whichever part is last) and
-// returns true.  Nobody waits for anybody.  `lds_flag` is a word of LDS no copy is in flight to.
+// index fastest; only the NTF live fragments of the groups that have rows), makes them visible to the
+// device and counts itself in; the part that counts last adds all parts in part order (its own too,
+// from memory: the same bits whichever part is last) and returns true.  Nobody waits for anybody.
+// `lds_flag` is a word of LDS no copy is in flight to.
 constexpr int kUpTailJobs = 64;
-__device__ __forceinline__ bool join_parts(const MoeArgs &a, const Job &j, f32x16 (&acc)[2][4], int *lds_flag) {
+template <int NTF>
+__device__ __forceinline__ bool join_parts(const MoeArgs &a, const Job &j, f32x16 (&acc)[2][4], bool active,
+                                           int *lds_flag) {
     const int tid = threadIdx.x;
     float4 *mine = reinterpret_cast<float4 *>(a.up_partials) + ((int64_t)(j.slot * 4 + j.part) * 32) * 512;
+    if (active) {
 #pragma unroll
-    for (int f = 0; f < 2; ++f)
+        for (int f = 0; f < 2; ++f)
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < NTF; ++t)
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-                mine[((f * 4 + t) * 4 + q) * 512 + tid] =
-                    make_float4(acc[f][t][4 * q], acc[f][t][4 * q + 1], acc[f][t][4 * q + 2], acc[f][t][4 * q + 3]);
+                for (int q = 0; q < 4; ++q)
+                    mine[((f * 4 + t) * 4 + q) * 512 + tid] =
+                        make_float4(acc[f][t][4 * q], acc[f][t][4 * q + 1], acc[f][t][4 * q + 2], acc[f][t][4 * q + 3]);
+    }
     __threadfence();  // the stores above are visible device-wide before the count below
     __syncthreads();
     if (tid == 0) *lds_flag = atomicAdd(&a.up_counters[j.slot], 1);
@@ -317,21 +322,23 @@ __device__ __forceinline__ bool join_parts(const MoeArgs &a, const Job &j, f32x1
     const bool last = *lds_flag == j.parts - 1;
     if (!last) return false;
     __threadfence();  // the other parts' stores are visible to the loads below
-    zero_acc(acc);
-    for (int p = 0; p < j.parts; ++p) {
-        const float4 *src = reinterpret_cast<const float4 *>(a.up_partials) + ((int64_t)(j.slot * 4 + p) * 32) * 512;
+    if (active) {
+        zero_acc(acc);
+        for (int p = 0; p < j.parts; ++p) {
+            const float4 *src = reinterpret_cast<const float4 *>(a.up_partials) + ((int64_t)(j.slot * 4 + p) * 32) * 512;
 #pragma unroll
-        for (int f = 0; f < 2; ++f)
+            for (int f = 0; f < 2; ++f)
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+                for (int t = 0; t < NTF; ++t)
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float4 v = src[((f * 4 + t) * 4 + q) * 512 + tid];
-                    acc[f][t][4 * q] += v.x;
-                    acc[f][t][4 * q + 1] += v.y;
-                    acc[f][t][4 * q + 2] += v.z;
-                    acc[f][t][4 * q + 3] += v.w;
-                }
+                    for (int q = 0; q < 4; ++q) {
+                        const float4 v = src[((f * 4 + t) * 4 + q) * 512 + tid];
+                        acc[f][t][4 * q] += v.x;
+                        acc[f][t][4 * q + 1] += v.y;
+                        acc[f][t][4 * q + 2] += v.z;
+                        acc[f][t][4 * q + 3] += v.w;
+                    }
+        }
     }
     return true;
 }
@@ -476,7 +483,7 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, const Job &job, R
         else
             ring::main_loop<DT, RB, NTF, true, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
         if constexpr (DT == DT_BF16) {
-            if (job.parts > 1 && !join_parts(a, job, acc, reinterpret_cast<int *>(lds + 128 * 1024))) return;
+            if (job.parts > 1 && !join_parts<NTF>(a, job, acc, active, reinterpret_cast<int *>(lds + 128 * 1024))) return;
         }
         const bool more = sub + 1 < n_sub;
         if (more) {
@@ -546,7 +553,7 @@ __device__ __forceinline__ void up_tile_wide_bf16(const MoeArgs &a, const Job &j
     if (active) ring128::main_loop<NTF, true, true>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
     else ring128::main_loop<NTF, true, false>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
     if constexpr (SPLIT) {
-        if (!join_parts(a, job, acc, reinterpret_cast<int *>(lds + 4 * ring128::kUnitBytes))) return;
+        if (!join_parts<NTF>(a, job, acc, active, reinterpret_cast<int *>(lds + 4 * ring128::kUnitBytes))) return;
     }
 
     char *tile = lds + grp * (kBlockRows * kActPitchBf16);

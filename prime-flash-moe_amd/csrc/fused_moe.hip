@@ -315,13 +315,13 @@ __device__ __forceinline__ bool join_parts(const MoeArgs &a, const Job &j, f32x1
                     mine[((f * 4 + t) * 4 + q) * 512 + tid] =
                         make_float4(acc[f][t][4 * q], acc[f][t][4 * q + 1], acc[f][t][4 * q + 2], acc[f][t][4 * q + 3]);
     }
-    __threadfence();  // the stores above are visible device-wide before the count below
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // the stores above are visible device-wide before the count below
     __syncthreads();
     if (tid == 0) *lds_flag = atomicAdd(&a.up_counters[j.slot], 1);
     __syncthreads();
     const bool last = *lds_flag == j.parts - 1;
     if (!last) return false;
-    __threadfence();  // the other parts' stores are visible to the loads below
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // the other parts' stores are visible to the loads below
     if (active) {
         zero_acc(acc);
         for (int p = 0; p < j.parts; ++p) {

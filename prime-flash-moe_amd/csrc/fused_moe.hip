@@ -45,8 +45,6 @@ struct MoeArgs {
     uint32_t *act_scales; // scales of the activation (written by the up kernel's epilogue)
     char *y;              // (sorted_num, K) bf16: down-projected rows, before the routing weights
     int32_t *inv;         // (M * top_k): sorted row of each pair id (validated against sorted_ids when read)
-    const int2 *tiles;    // row tiles built by the prologue: (first block, number of blocks 1..2)
-    const int *n_tiles;   // number of row tiles
     const int4 *work;     // this kernel's work list, one entry per workgroup (see emit_work)
     char *y_tail;         // partial tiles of down jobs whose contraction is split (see plan_tail_split)
     float *up_partials;   // fp32 partial accumulators of up jobs whose contraction is split
@@ -1089,8 +1087,6 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
     const int mask = g_phase_mask;
     a.n_blocks = (a.sorted_num + kBlockRows - 1) / kBlockRows;
     a.n_wtiles = a.H / 128;
-    a.tiles = sb.tiles;
-    a.n_tiles = sb.n_tiles;
     const int n_wt_down = (a.K + kWRows - 1) / kWRows;
     const int per_up = tiles_per_workgroup(DT, false, a.n_blocks, a.n_wtiles);
     const int per_down = tiles_per_workgroup(DT, true, a.n_blocks, n_wt_down);

@@ -39,6 +39,21 @@ def _require(cond: bool, msg: str) -> None:
     if not cond:
         raise RuntimeError(msg)
 
+def _require_same_device(what: str, named: dict, anchor: str = "x") -> None:
+    """Every tensor must live on the GPU of `anchor`: the kernels take raw device pointers, so a CPU
+    tensor (or one on another GPU) would be a memory fault on the device, not an exception."""
+    dev = named[anchor].device
+    _require(dev.type == "cuda", f"{what}: {anchor} must be a GPU tensor, got device {dev}")
+    for name, t in named.items():
+        _require(t.device == dev, f"{what}: {name} is on {t.device}, expected {dev} (the device of {anchor})")
+
+
+def _require_aligned(what: str, named: dict, names, align: int) -> None:
+    """The kernels read these with `align`-byte vector loads from the start of the tensor."""
+    for name in names:
+        _require(named[name].data_ptr() % align == 0,
+                 f"{what}: {name} must start at a {align}-byte aligned address")
+
 
 def _stream_ptr(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
@@ -59,6 +74,7 @@ def align_sizes(n: int, num_experts: int, block_m: int, bpc: int):
 
 
 def _validate_align(topk_ids: torch.Tensor, num_experts: int, block_m: int, bpc: int) -> None:
+    _require(topk_ids.is_cuda, f"moe_align: topk_ids must be a GPU tensor, got device {topk_ids.device}")
     _require(topk_ids.is_contiguous(), "moe_align: topk_ids must be contiguous")
     _require(topk_ids.dtype == torch.int32, "moe_align: topk_ids must be int32")
     _require(block_m > 0 and bpc > 0 and num_experts > 0, "moe_align: block_m, bpc and num_experts must be positive")
@@ -115,8 +131,12 @@ def _validate_bf16(x, w, w2, sorted_token_ids, expert_ids, num_tokens_post_padde
     _require(top_k > 0, "fused_moe_bf16: top_k must be positive")
     named = dict(x=x, w=w, w2=w2, sorted_token_ids=sorted_token_ids, expert_ids=expert_ids,
                  num_tokens_post_padded=num_tokens_post_padded, topk_weights=topk_weights, out=out)
+    _require_same_device("fused_moe_bf16", named)
     for name, t in named.items():
         _require(t.is_contiguous(), f"fused_moe_bf16: {name} must be contiguous")
+    _require_aligned("fused_moe_bf16", named, ("x", "w", "w2", "out"), 16)
+    _require_aligned("fused_moe_bf16", named, ("sorted_token_ids", "expert_ids", "num_tokens_post_padded",
+                                               "topk_weights"), 4)
     for name in ("x", "w", "w2", "out"):
         _require(named[name].dtype == torch.bfloat16, f"fused_moe_bf16: {name} must be bfloat16")
     _require(topk_weights.dtype == torch.float32, "fused_moe_bf16: topk_weights must be float32")
@@ -176,8 +196,12 @@ def _validate_mxfp8(x, x_scales, w, w_scales, w2, w2_scales, sorted_token_ids, e
     named = dict(x=x, x_scales=x_scales, w=w, w_scales=w_scales, w2=w2, w2_scales=w2_scales,
                  sorted_token_ids=sorted_token_ids, expert_ids=expert_ids,
                  num_tokens_post_padded=num_tokens_post_padded, topk_weights=topk_weights, out=out)
+    _require_same_device("fused_moe_mxfp8", named)
     for name, t in named.items():
         _require(t.is_contiguous(), f"fused_moe_mxfp8: {name} must be contiguous")
+    _require_aligned("fused_moe_mxfp8", named, ("x", "w", "w2", "out"), 16)
+    _require_aligned("fused_moe_mxfp8", named, ("x_scales", "w_scales", "w2_scales", "sorted_token_ids", "expert_ids",
+                                                "num_tokens_post_padded", "topk_weights"), 4)
     for name in ("x", "w", "w2"):
         _require(named[name].dtype == torch.float8_e4m3fn, f"fused_moe_mxfp8: {name} must be float8_e4m3fn")
     for name in ("x_scales", "w_scales", "w2_scales"):

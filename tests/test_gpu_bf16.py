@@ -135,6 +135,17 @@ def test_validation_errors(device):
         call(x=x.t().contiguous().t())
     with pytest.raises(RuntimeError):
         call(x=x[:, :192].contiguous())
+    # a tensor that is not on x's GPU is rejected on the host (its pointer never reaches a kernel)
+    with pytest.raises(RuntimeError, match="is on cpu"):
+        call(wts=wts.cpu())
+    with pytest.raises(RuntimeError, match="is on cpu"):
+        call(out=out.cpu())
+    with pytest.raises(RuntimeError, match="is on cpu"):
+        prime_moe.fused_moe_bf16(x, w1, w2, sched[0].cpu(), sched[1], sched[2], wts, out, top_k, 128, 64, 4, 2, 1, 1, True)
+    # x starting 2 bytes into an allocation: the 16-byte copies of the loaders would be misaligned
+    shifted = torch.empty((T * K + 1,), dtype=torch.bfloat16, device=device)[1:].view(T, K)
+    with pytest.raises(RuntimeError, match="aligned"):
+        call(x=shifted)
 
 
 def test_result_is_bitwise_reproducible(device):

@@ -112,6 +112,16 @@ def test_validation_errors(device):
         call(xs=a["x_scales"][:, :4].contiguous())
     with pytest.raises(RuntimeError):
         call(w1s=a["w1_scales"].reshape(-1)[:-1].contiguous())
+    # tensors that are not on x's GPU are rejected on the host (their pointers never reach a kernel)
+    with pytest.raises(RuntimeError, match="is on cpu"):
+        call(xs=a["x_scales"].cpu())
+    with pytest.raises(RuntimeError, match="is on cpu"):
+        call(w1s=a["w1_scales"].cpu())
+    # x scales starting 1 byte into an allocation: the kernels read them as 32-bit words
+    n_xs = a["x_scales"].numel()
+    shifted = torch.empty((n_xs + 1,), dtype=torch.uint8, device=device)[1:].view(torch.float8_e8m0fnu).view(T, K // 32)
+    with pytest.raises(RuntimeError, match="aligned"):
+        call(xs=shifted)
 
 
 @pytest.mark.parametrize("per", [2, 3, 16])

@@ -66,6 +66,23 @@ int pmoe_moe_align_ws(const int32_t *topk_ids, int32_t *sorted_token_ids, int32_
                       size_t workspace_bytes, void *stream);
 
 /*
+ * The same sort for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc); no counterpart in the reference.
+ * Takes what pmoe_moe_align takes and gives the same output, bit for bit, but the scratch of
+ * the multi-workgroup sort lives in a device array built into the library (516 KB on every
+ * device the library runs on, held until the process ends), so large inputs still spread
+ * over many workgroups.  n > PMOE_ALIGN_STATIC_MAX_IDS is rejected (PMOE_ERR_INVALID).
+ * Calls no hipMalloc / hipFree or any allocating routine; the first call on a device looks
+ * up the array's address (hipGetSymbolAddress), so make that one outside a capture.
+ * All calls on one device share the array: calls that overlap on one device (two streams,
+ * two threads) race and must be serialised by the caller.
+ */
+#define PMOE_ALIGN_STATIC_MAX_IDS (1 << 20)
+int pmoe_moe_align_static(const int32_t *topk_ids, int32_t *sorted_token_ids, int32_t *expert_ids,
+                          int32_t *num_tokens_post_padded, int n, int num_experts, int block_m,
+                          int pad_to, int max_padded, int max_blocks, void *stream);
+
+/*
  * Workspace (bytes) the fused calls below need for a problem of this size.  The
  * caller allocates it on the device (any 256-byte aligned buffer) and passes it in.
  * The size does not depend on `split` (both values run the same kernels); the argument

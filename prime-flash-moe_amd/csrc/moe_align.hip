@@ -11,6 +11,8 @@
 //      that group is a popcount of the lower lanes, and the destination is
 //      offs[e] + base[wave][e] + rank.
 // All arithmetic is int32 and the output is a pure function of the input.
+#include <mutex>
+
 #include "pmoe_common.h"
 
 namespace {
@@ -291,6 +293,109 @@ __global__ __launch_bounds__(NW * 64) void align_scatter_kernel(const int32_t *_
     }
 }
 
+
+// Scratch of the entry point that allocates nothing (pmoe_moe_align_static): counts[G][E], offs[E + 1],
+// cnt[E] of the multi-workgroup sort for up to kStaticMaxIds ids and kMaxExperts experts, 516 KB held by
+// every device the library runs on until the process ends.  In host code this name is only a handle for
+// hipGetSymbolAddress; kernels get the address that call returns.
+constexpr int kStaticMaxIds = PMOE_ALIGN_STATIC_MAX_IDS;
+constexpr size_t kStaticWords = (size_t)(kStaticMaxIds / kSliceIds) * kMaxExperts + 2 * kMaxExperts + 1;
+static __device__ __align__(256) int32_t scratch[kStaticWords];
+
+int id_bits_for(int num_experts) {
+    int id_bits = 1;
+    while ((1 << id_bits) < num_experts) ++id_bits;
+    return id_bits;
+}
+
+int validate(const int32_t *topk_ids, const int32_t *sorted_token_ids, const int32_t *expert_ids,
+             const int32_t *num_tokens_post_padded, int n, int num_experts, int block_m, int pad_to, int max_padded,
+             int max_blocks) {
+    PMOE_REQUIRE(num_experts > 0 && block_m > 0 && pad_to > 0, "moe_align: block_m, bpc and num_experts must be positive");
+    PMOE_REQUIRE(num_experts <= kMaxExperts, "moe_align supports at most 1024 experts, got %d", num_experts);
+    PMOE_REQUIRE(n >= 0 && max_padded >= 0 && max_blocks >= 0, "moe_align: negative size");
+    PMOE_REQUIRE(pad_to % block_m == 0, "moe_align: pad_to must be a multiple of block_m");
+    const long long need = ((long long)n + (long long)num_experts * (pad_to - 1) + pad_to - 1) / pad_to * pad_to;
+    PMOE_REQUIRE(max_padded >= need, "moe_align: max_padded %d is smaller than the worst case %lld", max_padded, need);
+    PMOE_REQUIRE((long long)max_blocks * block_m <= (long long)max_padded + block_m - 1,
+                 "moe_align: max_blocks %d does not match max_padded %d", max_blocks, max_padded);
+    PMOE_REQUIRE(sorted_token_ids && expert_ids && num_tokens_post_padded && (topk_ids || n == 0), "moe_align: null pointer");
+    return PMOE_OK;
+}
+
+// One workgroup sorts everything.
+int launch_single(const int32_t *topk_ids, int32_t *sorted_token_ids, int32_t *expert_ids,
+                  int32_t *num_tokens_post_padded, int n, int num_experts, int block_m, int pad_to, int max_padded,
+                  int max_blocks, hipStream_t s) {
+    const int id_bits = id_bits_for(num_experts);
+    if (num_experts <= 512) {
+        constexpr int NW = 16;
+        const size_t smem = sizeof(int32_t) * (size_t)(2 * num_experts + 1 + NW * num_experts);
+        hipLaunchKernelGGL(moe_align_kernel<NW>, dim3(1), dim3(NW * 64), smem, s, topk_ids, sorted_token_ids,
+                           expert_ids, num_tokens_post_padded, n, num_experts, block_m, pad_to, max_padded,
+                           max_blocks, id_bits);
+    } else {
+        constexpr int NW = 8;
+        const size_t smem = sizeof(int32_t) * (size_t)(2 * num_experts + 1 + NW * num_experts);
+        hipLaunchKernelGGL(moe_align_kernel<NW>, dim3(1), dim3(NW * 64), smem, s, topk_ids, sorted_token_ids,
+                           expert_ids, num_tokens_post_padded, n, num_experts, block_m, pad_to, max_padded,
+                           max_blocks, id_bits);
+    }
+    return pmoe::check_launch("moe_align launch");
+}
+
+// The three launches of the multi-workgroup sort; `words` holds G * E + 2 E + 1 int32 of device scratch,
+// every one of which is written before it is read.
+int launch_multi(const int32_t *topk_ids, int32_t *sorted_token_ids, int32_t *expert_ids,
+                 int32_t *num_tokens_post_padded, int n, int num_experts, int block_m, int pad_to, int max_padded,
+                 int max_blocks, int32_t *words, hipStream_t s) {
+    const int id_bits = id_bits_for(num_experts);
+    const int G = (n + kSliceIds - 1) / kSliceIds;
+    AlignScratch sc;
+    sc.counts = words;
+    sc.offs = sc.counts + (size_t)G * num_experts;
+    sc.cnt = sc.offs + num_experts + 1;
+    hipLaunchKernelGGL(align_count_kernel, dim3(G), dim3(1024), sizeof(int32_t) * num_experts, s, topk_ids, n,
+                       num_experts, sc.counts);
+    hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(1024), sizeof(int32_t) * (2 * num_experts + 1), s, sc, G,
+                       num_experts, block_m, pad_to, max_blocks, expert_ids, num_tokens_post_padded);
+    if (num_experts <= 512) {
+        constexpr int NW = 16;
+        hipLaunchKernelGGL(align_scatter_kernel<NW>, dim3(G), dim3(NW * 64),
+                           sizeof(int32_t) * (size_t)(2 * num_experts + 1 + NW * num_experts), s, topk_ids,
+                           sorted_token_ids, sc, n, num_experts, max_padded, id_bits);
+    } else {
+        constexpr int NW = 8;
+        hipLaunchKernelGGL(align_scatter_kernel<NW>, dim3(G), dim3(NW * 64),
+                           sizeof(int32_t) * (size_t)(2 * num_experts + 1 + NW * num_experts), s, topk_ids,
+                           sorted_token_ids, sc, n, num_experts, max_padded, id_bits);
+    }
+    return pmoe::check_launch("moe_align launch");
+}
+
+// Device address of `scratch` on the current device: every device holds its own copy of the array at
+// its own address, looked up once per device (with that device current) and kept.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+int32_t *g_scratch_ptr[kMaxDevices] = {nullptr};
+
+int static_scratch(int32_t **out) {
+    int dev = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return pmoe::fail(PMOE_ERR_HIP, "moe_align_static: hipGetDevice: %s", hipGetErrorString(err));
+    PMOE_REQUIRE(dev >= 0 && dev < kMaxDevices, "moe_align_static: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *p = nullptr;
+        err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || p == nullptr)
+            return pmoe::fail(PMOE_ERR_HIP, "moe_align_static: hipGetSymbolAddress: %s", hipGetErrorString(err));
+        g_scratch_ptr[dev] = static_cast<int32_t *>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return PMOE_OK;
+}
+
 }  // namespace
 
 extern "C" size_t pmoe_moe_align_workspace_bytes(int n, int num_experts) {
@@ -311,56 +416,33 @@ extern "C" int pmoe_moe_align_ws(const int32_t *topk_ids, int32_t *sorted_token_
                                  int32_t *num_tokens_post_padded, int n, int num_experts, int block_m, int pad_to,
                                  int max_padded, int max_blocks, void *workspace, size_t workspace_bytes,
                                  void *stream) {
-    PMOE_REQUIRE(num_experts > 0 && block_m > 0 && pad_to > 0, "moe_align: block_m, bpc and num_experts must be positive");
-    PMOE_REQUIRE(num_experts <= kMaxExperts, "moe_align supports at most 1024 experts, got %d", num_experts);
-    PMOE_REQUIRE(n >= 0 && max_padded >= 0 && max_blocks >= 0, "moe_align: negative size");
-    PMOE_REQUIRE(pad_to % block_m == 0, "moe_align: pad_to must be a multiple of block_m");
-    {
-        const long long need = ((long long)n + (long long)num_experts * (pad_to - 1) + pad_to - 1) / pad_to * pad_to;
-        PMOE_REQUIRE(max_padded >= need, "moe_align: max_padded %d is smaller than the worst case %lld", max_padded, need);
-        PMOE_REQUIRE((long long)max_blocks * block_m <= (long long)max_padded + block_m - 1, "moe_align: max_blocks %d does not match max_padded %d", max_blocks, max_padded);
-    }
-    PMOE_REQUIRE(sorted_token_ids && expert_ids && num_tokens_post_padded && (topk_ids || n == 0), "moe_align: null pointer");
-    int id_bits = 1;
-    while ((1 << id_bits) < num_experts) ++id_bits;
+    if (int rc = validate(topk_ids, sorted_token_ids, expert_ids, num_tokens_post_padded, n, num_experts, block_m,
+                          pad_to, max_padded, max_blocks))
+        return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const size_t ws_need = pmoe_moe_align_workspace_bytes(n, num_experts);
     if (ws_need > 0 && workspace != nullptr && workspace_bytes >= ws_need) {
         PMOE_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 3) == 0, "moe_align: workspace must be 4-byte aligned");
-        const int G = (n + kSliceIds - 1) / kSliceIds;
-        AlignScratch sc;
-        sc.counts = static_cast<int32_t *>(workspace);
-        sc.offs = sc.counts + (size_t)G * num_experts;
-        sc.cnt = sc.offs + num_experts + 1;
-        hipLaunchKernelGGL(align_count_kernel, dim3(G), dim3(1024), sizeof(int32_t) * num_experts, s, topk_ids, n,
-                           num_experts, sc.counts);
-        hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(1024), sizeof(int32_t) * (2 * num_experts + 1), s, sc, G,
-                           num_experts, block_m, pad_to, max_blocks, expert_ids, num_tokens_post_padded);
-        if (num_experts <= 512) {
-            constexpr int NW = 16;
-            hipLaunchKernelGGL(align_scatter_kernel<NW>, dim3(G), dim3(NW * 64),
-                               sizeof(int32_t) * (size_t)(2 * num_experts + 1 + NW * num_experts), s, topk_ids,
-                               sorted_token_ids, sc, n, num_experts, max_padded, id_bits);
-        } else {
-            constexpr int NW = 8;
-            hipLaunchKernelGGL(align_scatter_kernel<NW>, dim3(G), dim3(NW * 64),
-                               sizeof(int32_t) * (size_t)(2 * num_experts + 1 + NW * num_experts), s, topk_ids,
-                               sorted_token_ids, sc, n, num_experts, max_padded, id_bits);
-        }
-        return pmoe::check_launch("moe_align launch");
+        return launch_multi(topk_ids, sorted_token_ids, expert_ids, num_tokens_post_padded, n, num_experts, block_m,
+                            pad_to, max_padded, max_blocks, static_cast<int32_t *>(workspace), s);
     }
-    if (num_experts <= 512) {
-        constexpr int NW = 16;
-        size_t smem = sizeof(int32_t) * (size_t)(2 * num_experts + 1 + NW * num_experts);
-        hipLaunchKernelGGL(moe_align_kernel<NW>, dim3(1), dim3(NW * 64), smem, s, topk_ids,
-                           sorted_token_ids, expert_ids, num_tokens_post_padded, n, num_experts,
-                           block_m, pad_to, max_padded, max_blocks, id_bits);
-    } else {
-        constexpr int NW = 8;
-        size_t smem = sizeof(int32_t) * (size_t)(2 * num_experts + 1 + NW * num_experts);
-        hipLaunchKernelGGL(moe_align_kernel<NW>, dim3(1), dim3(NW * 64), smem, s, topk_ids,
-                           sorted_token_ids, expert_ids, num_tokens_post_padded, n, num_experts,
-                           block_m, pad_to, max_padded, max_blocks, id_bits);
-    }
-    return pmoe::check_launch("moe_align launch");
+    return launch_single(topk_ids, sorted_token_ids, expert_ids, num_tokens_post_padded, n, num_experts, block_m,
+                         pad_to, max_padded, max_blocks, s);
+}
+
+extern "C" int pmoe_moe_align_static(const int32_t *topk_ids, int32_t *sorted_token_ids, int32_t *expert_ids,
+                                     int32_t *num_tokens_post_padded, int n, int num_experts, int block_m,
+                                     int pad_to, int max_padded, int max_blocks, void *stream) {
+    if (int rc = validate(topk_ids, sorted_token_ids, expert_ids, num_tokens_post_padded, n, num_experts, block_m,
+                          pad_to, max_padded, max_blocks))
+        return rc;
+    PMOE_REQUIRE(n <= kStaticMaxIds, "moe_align_static: at most %d ids fit the built-in scratch, got %d", kStaticMaxIds, n);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (n <= kSingleMaxIds)  // one workgroup sorts these in its LDS: no device scratch involved
+        return launch_single(topk_ids, sorted_token_ids, expert_ids, num_tokens_post_padded, n, num_experts, block_m,
+                             pad_to, max_padded, max_blocks, s);
+    int32_t *words = nullptr;
+    if (int rc = static_scratch(&words)) return rc;
+    return launch_multi(topk_ids, sorted_token_ids, expert_ids, num_tokens_post_padded, n, num_experts, block_m,
+                        pad_to, max_padded, max_blocks, words, s);
 }

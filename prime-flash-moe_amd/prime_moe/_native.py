@@ -22,6 +22,7 @@ SIGNATURES = {
     "pmoe_moe_align": (_c_int, [_c_void_p] * 4 + [_c_int] * 6 + [_c_void_p]),
     "pmoe_moe_align_workspace_bytes": (_c_size_t, [_c_int] * 2),
     "pmoe_moe_align_ws": (_c_int, [_c_void_p] * 4 + [_c_int] * 6 + [_c_void_p, _c_size_t, _c_void_p]),
+    "pmoe_moe_align_static": (_c_int, [_c_void_p] * 4 + [_c_int] * 6 + [_c_void_p]),
     "pmoe_fused_moe_bf16_workspace_bytes": (_c_size_t, [_c_int] * 7),
     "pmoe_fused_moe_mxfp8_workspace_bytes": (_c_size_t, [_c_int] * 7),
     "pmoe_fused_moe_bf16": (_c_int, [_c_void_p] * 8 + [_c_int] * 13 + [_c_void_p, _c_size_t, _c_void_p]),

@@ -84,10 +84,10 @@ __device__ __forceinline__ uint32_t lds_addr(const char *p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
 }
 __device__ __forceinline__ void copy16(const char *base, uint32_t voff, const char *lds_dst) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr(lds_dst)) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr(lds_dst)) : "memory", "m0");
 }
 __device__ __forceinline__ void copy4(const char *base, uint32_t voff, const char *lds_dst) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr(lds_dst)) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr(lds_dst)) : "memory", "m0");
 }
 // A wave-uniform pointer, read through lane 0 so that the compiler keeps it in scalar registers.
 __device__ __forceinline__ const char *uniform_ptr(const char *p) {

@@ -147,31 +147,27 @@ int pmoe_quantize_mx(const void *src_bf16, void *q, void *scales, int64_t rows, 
                      void *stream);
 
 /*
- * Profiling aid with no counterpart in the reference: restricts, for the calling thread, which
- * kernels the two fused entry points enqueue, so a harness can time one kernel of the pipeline
- * with events around the call.  Results are only meaningful with PMOE_PHASE_ALL (the default).
+ * route -- the step in front of moe_align, which the reference leaves to the caller ("routing
+ * comes from your gate", README.md:147-149; its benchmark draws expert ids directly,
+ * benchmark/benchmark.py:124-166): gate logits -> top-k + softmax -> moe_align, enqueued
+ * back to back on `stream` with no host synchronisation.
+ *   logits (n_tokens, num_experts) fp32 or bf16 (logits_dtype), row major; bias (num_experts)
+ *   fp32 added to every row before the selection, or null.
+ *   topk_ids (n_tokens, top_k) int32: experts of the top_k largest values, largest first, ties
+ *   to the lower index, NaN above every number; topk_weights (n_tokens, top_k) fp32: softmax
+ *   over the selected values.  top_k <= min(32, num_experts), num_experts <= 1024.
+ *   sorted_token_ids / expert_ids / num_tokens_post_padded and the sizes that follow are those
+ *   of pmoe_moe_align_ws for n = n_tokens * top_k (workspace from
+ *   pmoe_moe_align_workspace_bytes(n, num_experts)); with sorted_token_ids == NULL only the
+ *   top-k and the weights are computed.
  */
-#define PMOE_PHASE_PROLOGUE 1 /* inversion of the sorted order (the work lists are always built) */
-#define PMOE_PHASE_UP 2       /* gate/up GEMM + SwiGLU */
-#define PMOE_PHASE_DOWN 4     /* down GEMM */
-#define PMOE_PHASE_FINALIZE 8 /* routing-weight reduction into bf16 `out` */
-#define PMOE_PHASE_ALL 15
-void pmoe_set_phase_mask(int mask);
-
-/*
- * Tuning and test aid with no counterpart in the reference: the number of consecutive weight tiles
- * (1..16) one workgroup of the mxfp8 up and down kernels takes for its row tile, for the calling
- * thread; 0 (the default) lets every launch choose from its sizes.  The result does not depend on it.
- */
-void pmoe_set_tiles_per_workgroup(int n);
-
-/*
- * Second profiling aid without a counterpart in the reference: a plain device copy of `bytes`
- * bytes (multiple of 16) done by a kernel named copy_calibration_kernel.  Its known traffic
- * (bytes read, bytes written) scales the FETCH_SIZE / WRITE_SIZE hardware counters of a
- * counter-collection run that also contains the fused kernels.
- */
-int pmoe_copy_calibration(const void *src, void *dst, int64_t bytes, void *stream);
+#define PMOE_DTYPE_F32 0
+#define PMOE_DTYPE_BF16 1
+int pmoe_route(const void *logits, int logits_dtype, const float *bias, int32_t *topk_ids,
+               float *topk_weights, int32_t *sorted_token_ids, int32_t *expert_ids,
+               int32_t *num_tokens_post_padded, int n_tokens, int num_experts, int top_k,
+               int block_m, int pad_to, int max_padded, int max_blocks, void *workspace,
+               size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

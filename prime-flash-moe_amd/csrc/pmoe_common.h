@@ -6,6 +6,7 @@
 #include <cstdio>
 
 #include "../../include/prime_moe_hip.h"
+#include "../../include/prime_moe_hip_debug.h"
 
 namespace pmoe {
 

@@ -10,7 +10,8 @@ the conditions the reference's ``TORCH_CHECK``s reject (torch_interface.cpp:85-8
 :132-155, :208-241).
 
 Extras that the reference leaves to its callers: a fake impl for ``moe_align`` (so all
-three ops trace), and :func:`quantize_mx`, the OCP-MX quantiser in front of the mxfp8 op.
+three ops trace), :func:`quantize_mx`, the OCP-MX quantiser in front of the mxfp8 op, and
+:func:`route`, the router front-end (top-k + softmax + ``moe_align``) in front of both.
 """
 from __future__ import annotations
 
@@ -73,8 +74,8 @@ def align_sizes(n: int, num_experts: int, block_m: int, bpc: int):
     return pad_to, max_padded, max_padded // block_m
 
 
-def _validate_align(topk_ids: torch.Tensor, num_experts: int, block_m: int, bpc: int) -> None:
-    _require(topk_ids.is_cuda, f"moe_align: topk_ids must be a GPU tensor, got device {topk_ids.device}")
+def _validate_align(topk_ids: torch.Tensor, num_experts: int, block_m: int, bpc: int, placement: bool = True) -> None:
+    _require(topk_ids.is_cuda or not placement, f"moe_align: topk_ids must be a GPU tensor, got device {topk_ids.device}")
     _require(topk_ids.is_contiguous(), "moe_align: topk_ids must be contiguous")
     _require(topk_ids.dtype == torch.int32, "moe_align: topk_ids must be int32")
     _require(block_m > 0 and bpc > 0 and num_experts > 0, "moe_align: block_m, bpc and num_experts must be positive")
@@ -117,7 +118,9 @@ def _check_tuning(block_m, block_n, warp_n, stages, max_stages, what):
 
 
 def _validate_bf16(x, w, w2, sorted_token_ids, expert_ids, num_tokens_post_padded, topk_weights, out,
-                   top_k, block_m, block_n, warp_n, stages, bpc, cpc, split) -> None:
+                   top_k, block_m, block_n, warp_n, stages, bpc, cpc, split, placement: bool = True) -> None:
+    """Argument checks of the op.  `placement=False` skips the device and alignment checks (what is
+    left can then be exercised with CPU tensors)."""
     _require(x.dim() == 2 and w.dim() == 3 and w2.dim() == 3, "fused_moe_bf16: x must be 2-D, w and w2 3-D")
     _require(x.size(0) > 0, "fused_moe_bf16: x has no rows")
     _require(x.size(1) == w.size(2), "fused_moe_bf16: x.size(1) must equal w.size(2)")
@@ -131,12 +134,13 @@ def _validate_bf16(x, w, w2, sorted_token_ids, expert_ids, num_tokens_post_padde
     _require(top_k > 0, "fused_moe_bf16: top_k must be positive")
     named = dict(x=x, w=w, w2=w2, sorted_token_ids=sorted_token_ids, expert_ids=expert_ids,
                  num_tokens_post_padded=num_tokens_post_padded, topk_weights=topk_weights, out=out)
-    _require_same_device("fused_moe_bf16", named)
+    if placement:
+        _require_same_device("fused_moe_bf16", named)
+        _require_aligned("fused_moe_bf16", named, ("x", "w", "w2", "out"), 16)
+        _require_aligned("fused_moe_bf16", named, ("sorted_token_ids", "expert_ids", "num_tokens_post_padded",
+                                                   "topk_weights"), 4)
     for name, t in named.items():
         _require(t.is_contiguous(), f"fused_moe_bf16: {name} must be contiguous")
-    _require_aligned("fused_moe_bf16", named, ("x", "w", "w2", "out"), 16)
-    _require_aligned("fused_moe_bf16", named, ("sorted_token_ids", "expert_ids", "num_tokens_post_padded",
-                                               "topk_weights"), 4)
     for name in ("x", "w", "w2", "out"):
         _require(named[name].dtype == torch.bfloat16, f"fused_moe_bf16: {name} must be bfloat16")
     _require(topk_weights.dtype == torch.float32, "fused_moe_bf16: topk_weights must be float32")
@@ -177,7 +181,8 @@ def _fused_moe_bf16_fake(x, w, w2, sorted_token_ids, expert_ids, num_tokens_post
 
 def _validate_mxfp8(x, x_scales, w, w_scales, w2, w2_scales, sorted_token_ids, expert_ids,
                     num_tokens_post_padded, topk_weights, out, top_k, block_m, block_n, warp_n, stages,
-                    bpc, split) -> None:
+                    bpc, split, placement: bool = True) -> None:
+    """Argument checks of the op.  `placement=False` skips the device and alignment checks."""
     _require(x.dim() == 2 and w.dim() == 3 and w2.dim() == 3, "fused_moe_mxfp8: x must be 2-D, w and w2 3-D")
     M, K = x.shape
     E, N = w.size(0), w.size(1)
@@ -196,12 +201,13 @@ def _validate_mxfp8(x, x_scales, w, w_scales, w2, w2_scales, sorted_token_ids, e
     named = dict(x=x, x_scales=x_scales, w=w, w_scales=w_scales, w2=w2, w2_scales=w2_scales,
                  sorted_token_ids=sorted_token_ids, expert_ids=expert_ids,
                  num_tokens_post_padded=num_tokens_post_padded, topk_weights=topk_weights, out=out)
-    _require_same_device("fused_moe_mxfp8", named)
+    if placement:
+        _require_same_device("fused_moe_mxfp8", named)
+        _require_aligned("fused_moe_mxfp8", named, ("x", "w", "w2", "out"), 16)
+        _require_aligned("fused_moe_mxfp8", named, ("x_scales", "w_scales", "w2_scales", "sorted_token_ids",
+                                                    "expert_ids", "num_tokens_post_padded", "topk_weights"), 4)
     for name, t in named.items():
         _require(t.is_contiguous(), f"fused_moe_mxfp8: {name} must be contiguous")
-    _require_aligned("fused_moe_mxfp8", named, ("x", "w", "w2", "out"), 16)
-    _require_aligned("fused_moe_mxfp8", named, ("x_scales", "w_scales", "w2_scales", "sorted_token_ids", "expert_ids",
-                                                "num_tokens_post_padded", "topk_weights"), 4)
     for name in ("x", "w", "w2"):
         _require(named[name].dtype == torch.float8_e4m3fn, f"fused_moe_mxfp8: {name} must be float8_e4m3fn")
     for name in ("x_scales", "w_scales", "w2_scales"):
@@ -316,7 +322,49 @@ def quantize_mx(t: torch.Tensor):
     return q, s.view(torch.float8_e8m0fnu)
 
 
+def route(logits: torch.Tensor, top_k: int, block_m: int = 128, bpc: int = 1, bias: torch.Tensor = None):
+    """Router front-end: gate logits ``(T, E)`` -> top-k, softmax weights and the ``moe_align`` schedule.
+
+    The step the reference leaves to its callers (README.md:147-149): returns
+    ``(topk_ids (T, top_k) int32, topk_weights (T, top_k) fp32, sorted_token_ids, expert_ids,
+    num_tokens_post_padded)``; the last three are what ``torch.ops.prime_moe.moe_align(topk_ids, E,
+    block_m, bpc)`` returns.  Selection: the ``top_k`` largest of ``logits[t] (+ bias)``, largest first,
+    ties to the lower expert index; weights: softmax over the selected values in fp32.  One top-k kernel
+    plus the align kernels on the current stream, no host synchronisation.
+    """
+    _require(logits.is_cuda, f"route: logits must be a GPU tensor, got device {logits.device}")
+    _require(logits.dim() == 2 and logits.is_contiguous(), "route: logits must be a contiguous (T, E) tensor")
+    _require(logits.dtype in (torch.float32, torch.bfloat16), "route: logits must be float32 or bfloat16")
+    T, E = logits.shape
+    _require(0 < E <= 1024, f"route supports 1..1024 experts, got {E}")
+    _require(0 < top_k <= min(32, E), f"route: top_k must be in 1..min(32, E), got {top_k}")
+    _require(block_m > 0 and bpc > 0, "route: block_m and bpc must be positive")
+    if bias is not None:
+        _require(bias.device == logits.device and bias.dtype == torch.float32 and bias.is_contiguous()
+                 and bias.numel() == E, "route: bias must be a contiguous float32 (E,) tensor on the device of logits")
+    dev = logits.device
+    n = T * top_k
+    pad_to, max_padded, max_blocks = align_sizes(n, E, block_m, bpc)
+    topk_ids = torch.empty((T, top_k), dtype=torch.int32, device=dev)
+    topk_weights = torch.empty((T, top_k), dtype=torch.float32, device=dev)
+    sorted_token_ids = torch.empty((max_padded,), dtype=torch.int32, device=dev)
+    expert_ids = torch.empty((max_blocks,), dtype=torch.int32, device=dev)
+    num_tokens_post_padded = torch.empty((1,), dtype=torch.int32, device=dev)
+    lib = _native.load()
+    ws_bytes = lib.pmoe_moe_align_workspace_bytes(n, E)
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes else None
+    with torch.cuda.device(dev):
+        _native.check(lib.pmoe_route(
+            logits.data_ptr(), 0 if logits.dtype == torch.float32 else 1,
+            bias.data_ptr() if bias is not None else None, topk_ids.data_ptr(), topk_weights.data_ptr(),
+            sorted_token_ids.data_ptr(), expert_ids.data_ptr(), num_tokens_post_padded.data_ptr(), T, E, top_k,
+            block_m, pad_to, max_padded, max_blocks, ws.data_ptr() if ws is not None else None, ws_bytes,
+            _stream_ptr(dev)))
+    return topk_ids, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded
+
+
 __all__ = [
+    "route",
     "fused_moe_bf16",
     "fused_moe_mxfp8",
     "pack_scales_blocked",

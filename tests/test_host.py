@@ -16,7 +16,11 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def test_library_exports_every_declared_symbol():
     from prime_moe import _native
-    header = open(os.path.join(ROOT, "include", "prime_moe_hip.h")).read()
+    # the seam (prime_moe_hip.h) and the profiling / test hooks (prime_moe_hip_debug.h)
+    inc = os.path.join(ROOT, "include")
+    header = "".join(open(os.path.join(inc, f)).read() for f in sorted(os.listdir(inc)) if f.endswith(".h"))
+    seam = open(os.path.join(inc, "prime_moe_hip.h")).read()
+    assert "pmoe_set_phase_mask" not in seam and "pmoe_copy_calibration" not in seam
     declared = set(re.findall(r"\b(pmoe_[a-z0-9_]+)\s*\(", header))
     assert declared == set(_native.SIGNATURES), (declared, set(_native.SIGNATURES))
     lib = _native.load()
@@ -131,8 +135,10 @@ def _bf16_args(T=16, K=256, E=2, N=256, top_k=2):
 def test_bf16_validation_matrix():
     # conditions of the reference's TORCH_CHECKs (torch_interface.cpp:132-155)
     import prime_moe
-    v = prime_moe._validate_bf16
+    v = lambda *a: prime_moe._validate_bf16(*a, placement=False)  # CPU tensors: no device checks here
     v(*_bf16_args())
+    with pytest.raises(RuntimeError, match="must be a GPU tensor"):
+        prime_moe._validate_bf16(*_bf16_args())  # as the op calls it: a CPU tensor never reaches a kernel
     def bad(idx, val):
         a = _bf16_args()
         a[idx] = val
@@ -172,7 +178,9 @@ def test_mxfp8_validation_matrix():
             num_tokens_post_padded=torch.zeros((1,), dtype=torch.int32),
             topk_weights=torch.zeros((T, top_k), dtype=torch.float32), out=torch.zeros((T, K), dtype=torch.bfloat16),
             top_k=top_k, block_m=128, block_n=32, warp_n=8, stages=4, bpc=1, split=True)
-    prime_moe._validate_mxfp8(**args())
+    prime_moe._validate_mxfp8(**args(), placement=False)  # CPU tensors: no device checks here
+    with pytest.raises(RuntimeError, match="must be a GPU tensor"):
+        prime_moe._validate_mxfp8(**args())
     for key, val in [("block_m", 64), ("stages", 5), ("stages", 0), ("bpc", 2), ("warp_n", 4),
                      ("x", torch.zeros((T, K), dtype=torch.uint8)),
                      ("x_scales", torch.zeros((T, K // 32), dtype=torch.uint8)),
@@ -184,7 +192,7 @@ def test_mxfp8_validation_matrix():
         a = args()
         a[key] = val
         with pytest.raises(RuntimeError):
-            prime_moe._validate_mxfp8(**a)
+            prime_moe._validate_mxfp8(**a, placement=False)
 
 
 def test_align_validation_and_sizes():
@@ -194,11 +202,13 @@ def test_align_validation_and_sizes():
     assert prime_moe.align_sizes(10, 3, 24, 3) == (72, 288, 12)
     assert prime_moe.align_sizes(10, 3, 24, 3)[1:] == O.moe_align_sizes(10, 3, 24, 3)[1:]
     ok = torch.zeros((8,), dtype=torch.int32)
-    prime_moe._validate_align(ok, 4, 128, 1)
+    prime_moe._validate_align(ok, 4, 128, 1, placement=False)
+    with pytest.raises(RuntimeError, match="must be a GPU tensor"):
+        prime_moe._validate_align(ok, 4, 128, 1)
     for a in [(ok.long(), 4, 128, 1), (ok, 0, 128, 1), (ok, 4, 0, 1), (ok, 4, 128, 0), (ok, 1025, 128, 1),
               (torch.zeros((8, 2), dtype=torch.int32)[:, 0], 4, 128, 1)]:
         with pytest.raises(RuntimeError):
-            prime_moe._validate_align(*a)
+            prime_moe._validate_align(*a, placement=False)
 
 
 def test_ops_refuse_cpu_tensors():

@@ -31,6 +31,12 @@ reference checkout) and names the independent checks that pin it
                        Pinned by: dense per-token brute force in fp64, the
                        top_k=1/E=1 reduction to a plain SwiGLU MLP, token
                        permutation equivariance, duplicate-expert additivity.
+  route_topk           the routing the reference's callers do in front of moe_align
+                       (README.md:147-149): top-k of the gate logits by value,
+                       largest first, ties to the lower expert index, softmax over
+                       the selected values.
+                       Pinned by: torch.topk + torch.softmax on tie-free inputs, a
+                       hand-worked example with ties, weights summing to one.
 """
 from __future__ import annotations
 
@@ -118,6 +124,27 @@ def moe_align_fast(topk_ids, num_experts: int, block_m: int, bpc: int = 1):
     # experts with zero rows never own a block: searchsorted(right) skips them
     eid = np.where(rows >= total, num_experts - 1, np.minimum(eid, num_experts - 1))
     return sorted_ids, eid.astype(np.int32), np.array([total], dtype=np.int32)
+
+
+# --------------------------------------------------------------------------- routing
+
+def route_topk(logits: np.ndarray, top_k: int, bias: np.ndarray = None):
+    """Top-k routing in front of moe_align (what the reference's README.md:147-149 leaves to the gate).
+
+    ids[t, r] = expert of the r-th largest value of logits[t] (+ bias), ties to the lower index;
+    weights[t] = softmax over the selected values (float64 math, returned as float32).
+    The addition of the bias is done in float32, as a gate would.
+    """
+    v = np.asarray(logits, dtype=np.float32)
+    if bias is not None:
+        v = (v + np.asarray(bias, dtype=np.float32)[None, :]).astype(np.float32)
+    v = v + np.float32(0.0)  # -0 -> +0
+    order = np.argsort(-v.astype(np.float64), axis=1, kind="stable")  # stable: equal values keep index order
+    ids = order[:, :top_k]
+    sel = np.take_along_axis(v, ids, axis=1).astype(np.float64)
+    ex = np.exp(sel - sel[:, :1])
+    w = ex / ex.sum(axis=1, keepdims=True)
+    return ids.astype(np.int32), w.astype(np.float32)
 
 
 # --------------------------------------------------------------------------- scale packing

@@ -28,6 +28,7 @@ SIGNATURES = {
     "pmoe_fused_moe_bf16": (_c_int, [_c_void_p] * 8 + [_c_int] * 13 + [_c_void_p, _c_size_t, _c_void_p]),
     "pmoe_fused_moe_mxfp8": (_c_int, [_c_void_p] * 11 + [_c_int] * 12 + [_c_void_p, _c_size_t, _c_void_p]),
     "pmoe_quantize_mx": (_c_int, [_c_void_p] * 3 + [ctypes.c_int64, _c_int, _c_void_p]),
+    "pmoe_route": (_c_int, [_c_void_p, _c_int] + [_c_void_p] * 6 + [_c_int] * 7 + [_c_void_p, _c_size_t, _c_void_p]),
     "pmoe_set_phase_mask": (None, [_c_int]),
     "pmoe_set_tiles_per_workgroup": (None, [_c_int]),
     "pmoe_copy_calibration": (_c_int, [_c_void_p, _c_void_p, ctypes.c_int64, _c_void_p]),

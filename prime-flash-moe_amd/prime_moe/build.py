@@ -17,7 +17,7 @@ CSRC = os.path.join(os.path.dirname(HERE), "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_NAME = "libprime_moe_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["api.hip", "moe_align.hip", "quantize_mx.hip", "fused_moe.hip"]
+SOURCES = ["api.hip", "moe_align.hip", "route.hip", "quantize_mx.hip", "fused_moe.hip"]
 ARCH = "gfx950"
 
 # Packed-fp32 VALU forms are switched off for every device compile.

@@ -308,3 +308,33 @@ def test_forward_act_mx_matches_manual():
 
 def test_flops_model():
     assert O.approx_flops(4096, 2, 4096, 28672) == 3.0 * 8192 * 4096 * 28672
+
+
+# ----------------------------------------------------------------------------------- routing
+
+def test_route_topk_hand_example_with_ties():
+    # values: expert 1 and 3 tie at 2.0 (lower index first), then expert 0 and 4 tie at 1.0
+    logits = np.array([[1.0, 2.0, -1.0, 2.0, 1.0, 0.5]], dtype=np.float32)
+    ids, w = O.route_topk(logits, 3)
+    assert ids.tolist() == [[1, 3, 0]]
+    e = np.exp(np.array([0.0, 0.0, -1.0]))
+    np.testing.assert_allclose(w[0], e / e.sum(), rtol=1e-6)
+    ids, _ = O.route_topk(logits, 6)
+    assert ids.tolist() == [[1, 3, 0, 4, 5, 2]]
+    # -0 and +0 tie (lower index first); the bias is added before the selection
+    ids, _ = O.route_topk(np.array([[0.0, -0.0, -1.0]], dtype=np.float32), 2)
+    assert ids.tolist() == [[0, 1]]
+    ids, w = O.route_topk(np.array([[0.0, 0.0, 0.0]], dtype=np.float32), 1, bias=np.array([0.0, 0.0, 1.0]))
+    assert ids.tolist() == [[2]] and w.tolist() == [[1.0]]
+
+
+@pytest.mark.parametrize("T,E,k", [(64, 8, 2), (33, 128, 8), (5, 1000, 32), (7, 1, 1)])
+def test_route_topk_matches_torch_on_tie_free_inputs(T, E, k):
+    g = torch.Generator().manual_seed(T + E)
+    logits = torch.randn((T, E), generator=g)
+    assert all(torch.unique(row).numel() == E for row in logits)  # no ties: torch.topk's order is then unique
+    vals, idx = torch.topk(logits, k, dim=-1)
+    ids, w = O.route_topk(logits.numpy(), k)
+    np.testing.assert_array_equal(ids, idx.numpy().astype(np.int32))
+    np.testing.assert_allclose(w, torch.softmax(vals.float(), -1).numpy(), rtol=2e-6, atol=1e-7)
+    np.testing.assert_allclose(w.sum(1), 1.0, rtol=1e-6)

@@ -331,6 +331,36 @@ def fused_moe_dense(x, w1, w2, topk_ids, topk_weights, act_mx: bool = False,
     return out
 
 
+def fused_moe_by_expert(x, expert_weights, topk_ids, topk_weights, num_experts: int, act_mx: bool = False,
+                        experts=None, dtype=torch.float32) -> torch.Tensor:
+    """fused_moe_dense with the weights fetched one expert at a time: ``expert_weights(e)`` returns
+    ``(w1_e (2H, K), w2_e (K, H))`` (already dequantised for mxfp8) on the device of ``x``.  Keeps the
+    memory of a full-size configuration bounded, and runs wherever ``x`` lives.  ``experts``: only
+    these experts contribute (the pairs routed elsewhere add nothing), for checks on a subset.
+    Same dataflow and citations as fused_moe_dense; pinned against it in tests/test_oracle.py.
+    """
+    T, K = x.shape
+    xf = x.to(dtype)
+    out = torch.zeros((T, K), dtype=dtype, device=x.device)
+    ids = topk_ids.to(torch.int64)
+    wts = topk_weights.to(dtype)
+    todo = range(num_experts) if experts is None else sorted(int(e) for e in experts)
+    for e in todo:
+        tok, slot = torch.nonzero(ids == e, as_tuple=True)
+        if tok.numel() == 0:
+            continue
+        w1, w2 = expert_weights(e)
+        H = w1.shape[0] // 2
+        h = xf[tok] @ w1.to(dtype).t()
+        act = swiglu(h[:, :H], h[:, H:])
+        if act_mx:
+            q, s = quantize_mx_torch(act.float())
+            act = dequantize_mx_torch(q, s).to(dtype)
+        y = act @ w2.to(dtype).t()
+        out.index_add_(0, tok, y * wts[tok, slot][:, None])
+    return out
+
+
 def fused_moe_sorted(x, w1, w2, sorted_token_ids, expert_ids, num_tokens_post_padded,
                      topk_weights, top_k: int, block_m: int = 128, act_mx: bool = False,
                      act_bf16: bool = False, dtype=torch.float32) -> torch.Tensor:

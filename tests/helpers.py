@@ -7,6 +7,10 @@ from oracle import moe_oracle as O
 BF16_GATE = 2e-2        # max |got - ref| / max(|ref|, 1) for the bf16 path
 MX_COS_GATE = 0.999     # cosine similarity floor for the mxfp8 path
 MX_RELL2_GATE = 2e-2    # ||got - ref|| / ||ref|| ceiling for the mxfp8 path
+# element-wise gates of the mxfp8 path, the reference's own metric and values (test/test_mxfp8.py:14-15,
+# :168-191): max |got - ref| / max(|ref|, c) for c = 1 and c = 10
+MX_REL_CLAMP_1_GATE = 2e-2
+MX_REL_CLAMP_10_GATE = 2e-3
 
 
 def rel_clamp(got: torch.Tensor, ref: torch.Tensor, c: float) -> float:

@@ -1,25 +1,32 @@
 """fused_moe_mxfp8 on the GPU vs the fp32 CPU oracle evaluated on the dequantised inputs with
-the activation quantise->dequantise modelled.  Gates: cosine >= 0.999, rel-L2 <= 2e-2."""
+the activation quantise->dequantise modelled.  Gates: cosine >= 0.999, rel-L2 <= 2e-2 and, element
+by element, the reference's own metric and thresholds (test/test_mxfp8.py:14-15, :168-191):
+max |got - ref| / max(|ref|, 1) <= 2e-2 and max |got - ref| / max(|ref|, 10) <= 2e-3."""
 import math
+import os
 
 import numpy as np
 import pytest
 import torch
 
-from helpers import MX_COS_GATE, MX_RELL2_GATE, cosine, oracle_schedule, reference_routing, rel_clamp, rel_l2
+from helpers import (MX_COS_GATE, MX_REL_CLAMP_1_GATE, MX_REL_CLAMP_10_GATE, MX_RELL2_GATE, cosine, oracle_schedule,
+                     reference_routing, rel_clamp, rel_l2)
 from oracle import moe_oracle as O
 
 pytestmark = pytest.mark.gpu
 
 
-def _quantised_inputs(T, K, E, N, device, seed, x_std=1.0):
+def _quantised_inputs(T, K, E, N, device, seed, x_std=1.0, w_std=None):
     """bf16 masters on the device, quantised by the CPU oracle (so the op's inputs do not depend
-    on the GPU quantiser), packed with the product's pack_scales_blocked."""
+    on the GPU quantiser), packed with the product's pack_scales_blocked.  Weights ~ N(0, 1/fan_in)
+    unless `w_std` is given (the reference's tests draw x and the weights from N(0, 0.05^2),
+    test/test_mxfp8.py:118-123)."""
     import prime_moe
     g = torch.Generator(device=device).manual_seed(seed)
     x = (torch.randn((T, K), device=device, generator=g) * x_std).to(torch.bfloat16)
-    w1 = (torch.randn((E, N, K), device=device, generator=g) / math.sqrt(K)).to(torch.bfloat16)
-    w2 = (torch.randn((E, K, N // 2), device=device, generator=g) / math.sqrt(N // 2)).to(torch.bfloat16)
+    s1, s2 = (1 / math.sqrt(K), 1 / math.sqrt(N // 2)) if w_std is None else (w_std, w_std)
+    w1 = (torch.randn((E, N, K), device=device, generator=g) * s1).to(torch.bfloat16)
+    w2 = (torch.randn((E, K, N // 2), device=device, generator=g) * s2).to(torch.bfloat16)
     q = {}
     for name, t in (("x", x), ("w1", w1), ("w2", w2)):
         qt, st = O.quantize_mx_torch(t.float().cpu())
@@ -35,9 +42,10 @@ def _quantised_inputs(T, K, E, N, device, seed, x_std=1.0):
     return g, args, deq
 
 
-def _run_case(T, K, E, N, top_k, split, device, seed=0, use_op_align=True, exact=False, hot_last=True):
+def _run_case(T, K, E, N, top_k, split, device, seed=0, use_op_align=True, exact=False, hot_last=True,
+              x_std=1.0, w_std=None):
     import prime_moe
-    g, a, deq = _quantised_inputs(T, K, E, N, device, seed)
+    g, a, deq = _quantised_inputs(T, K, E, N, device, seed, x_std=x_std, w_std=w_std)
     ids, wts = reference_routing(T, E, top_k, device, g, hot_last=hot_last)
     sched = torch.ops.prime_moe.moe_align(ids, E, 128, 1) if use_op_align else oracle_schedule(ids, E, 128, exact)
     out = torch.zeros((T, K), dtype=torch.bfloat16, device=device) if not split else \
@@ -52,7 +60,35 @@ def _run_case(T, K, E, N, top_k, split, device, seed=0, use_op_align=True, exact
     c, l2 = cosine(got, ref), rel_l2(got, ref)
     assert c >= MX_COS_GATE, f"cosine {c}"
     assert l2 <= MX_RELL2_GATE, f"rel-L2 {l2}"
-    return c, l2
+    rc1, rc10, frac = _elementwise_gates(got, ref)
+    if os.environ.get("PMOE_PRINT_METRICS") == "1":
+        print(f"\nmxfp8 T={T} K={K} E={E} N={N} split={split}: cosine {c:.6f} rel-L2 {l2:.3g} rel_clamp_1 {rc1:.3g} "
+              f"rel_clamp_10 {rc10:.3g} rows beyond 2e-2: {frac:.4f}")
+    return c, l2, rc1, rc10
+
+
+def _elementwise_gates(got, ref):
+    """Element by element, in the reference's metric (test/test_mxfp8.py:168-191): a wrong scale byte or
+    K block of a weight row fails these, whatever the norms say.
+
+    The oracle and the kernel add the same fp32 products in different orders, so an activation that sits on
+    a rounding boundary of e4m3 can land on the neighbouring code in one of them: one token row then moves
+    by up to (code spacing) x |w2| x routing weight, a few 1e-2 for data of unit scale and a contraction as
+    short as H = 128.  Hence two tiers: every element within the loose gates (worst measured over the
+    reference's whole grid 6.7e-2 / 6.7e-3, gates 0.15 / 0.015), and all but 2 % of the token rows (at
+    least one row is allowed; worst measured over that grid 2 rows of 256) within the reference's own
+    thresholds of 2e-2 / 2e-3.
+    """
+    d = (got.double() - ref.double()).abs()
+    rc1 = float((d / ref.double().abs().clamp_min(1.0)).max())
+    rc10 = float((d / ref.double().abs().clamp_min(10.0)).max())
+    assert rc1 <= 0.15, f"rel_clamp_1 {rc1}"
+    assert rc10 <= 0.015, f"rel_clamp_10 {rc10}"
+    row1 = (d / ref.double().abs().clamp_min(1.0)).amax(1)
+    row10 = (d / ref.double().abs().clamp_min(10.0)).amax(1)
+    beyond = int(((row1 > MX_REL_CLAMP_1_GATE) | (row10 > MX_REL_CLAMP_10_GATE)).sum())
+    assert beyond <= max(1, got.shape[0] // 50), f"{beyond} of {got.shape[0]} token rows beyond the element-wise gates"
+    return rc1, rc10, beyond / got.shape[0]
 
 
 @pytest.mark.parametrize("split", [True, False])
@@ -63,6 +99,37 @@ def _run_case(T, K, E, N, top_k, split, device, seed=0, use_op_align=True, exact
 def test_reference_sweep_shapes(T, K, E, N, split, device):
     top_k = 9 if E > 1 else 1
     _run_case(T, K, E, N, top_k, split, device, seed=T + E)
+
+
+@pytest.mark.parametrize("split", [True, False])
+@pytest.mark.parametrize("T,K,E,N", [(256, 7168, 37, 512), (128, 4096, 257, 256), (32, 4096, 8, 512)])
+def test_reference_data_scales(T, K, E, N, split, device):
+    # x and weights ~ N(0, 0.05^2) as in the reference's own test (test/test_mxfp8.py:118-123), where
+    # |ref| << 1 makes both element-wise gates absolute ones (2e-2); it reports 3.3e-3 / 3.3e-4 for its
+    # kernel on this grid, the gates leave the same headroom here
+    _, _, rc1, rc10 = _run_case(T, K, E, N, 9, split, device, seed=3 * T + E, x_std=0.05, w_std=0.05)
+    assert rc1 <= 3.3e-3 and rc10 <= 3.3e-4, (rc1, rc10)
+
+
+def test_one_wrong_scale_byte_fails_the_elementwise_gate(device):
+    # the element-wise gate must see what the norm gates miss: flip one e8m0 scale of one weight row
+    # (one 32-wide K block of one row of one expert) and compare against the oracle on the intact data
+    import prime_moe
+    T, K, E, N, top_k = 128, 1024, 4, 512, 2
+    g, a, deq = _quantised_inputs(T, K, E, N, device, seed=77)
+    ids, wts = reference_routing(T, E, top_k, device, g, hot_last=False)
+    sched = torch.ops.prime_moe.moe_align(ids, E, 128, 1)
+    ref = O.fused_moe_dense(deq["x"], deq["w1"], deq["w2"], ids.cpu(), wts.cpu(), act_mx=True)
+    bad = a["w2_scales"].view(torch.uint8).clone()
+    bad.view(-1)[5] += 1  # scale x2 for one (row, 32-block) of expert 0's w2
+    out = torch.empty((T, K), dtype=torch.bfloat16, device=device)
+    prime_moe.fused_moe_mxfp8(a["x"], a["x_scales"], a["w1"], a["w1_scales"], a["w2"],
+                              bad.view(torch.float8_e8m0fnu), *sched, wts, out, top_k, 128, 64, 4, 2, 1, True)
+    torch.cuda.synchronize()
+    got = out.float().cpu()
+    assert cosine(got, ref) >= MX_COS_GATE and rel_l2(got, ref) <= MX_RELL2_GATE  # the norm gates do not notice
+    with pytest.raises(AssertionError):                                            # the element-wise ones do
+        _elementwise_gates(got, ref)
 
 
 @pytest.mark.parametrize("split", [True, False])

@@ -338,3 +338,16 @@ def test_route_topk_matches_torch_on_tie_free_inputs(T, E, k):
     np.testing.assert_array_equal(ids, idx.numpy().astype(np.int32))
     np.testing.assert_allclose(w, torch.softmax(vals.float(), -1).numpy(), rtol=2e-6, atol=1e-7)
     np.testing.assert_allclose(w.sum(1), 1.0, rtol=1e-6)
+
+
+def test_forward_by_expert_equals_dense_and_subset_masks():
+    x, w1, w2, ids, wts = _tiny(seed=9, T=12, K=16, E=5, H=32, k=3, dtype=torch.float32)
+    fetch = lambda e: (w1[e], w2[e])
+    for act_mx in (False, True):
+        dense = O.fused_moe_dense(x, w1, w2, ids, wts, act_mx=act_mx)
+        torch.testing.assert_close(O.fused_moe_by_expert(x, fetch, ids, wts, 5, act_mx=act_mx), dense, rtol=1e-6, atol=1e-6)
+        # a subset of experts == the dense result with the other pairs' routing weights zeroed
+        keep = (ids == 1) | (ids == 3)
+        masked = O.fused_moe_dense(x, w1, w2, ids, wts * keep, act_mx=act_mx)
+        torch.testing.assert_close(O.fused_moe_by_expert(x, fetch, ids, wts, 5, act_mx=act_mx, experts=[3, 1]),
+                                   masked, rtol=1e-6, atol=1e-6)

@@ -83,11 +83,14 @@ constexpr int ring_bytes() {
 __device__ __forceinline__ uint32_t lds_addr(const char *p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
 }
+// (M0 is written inside the statements without being declared: the compiler reserves the register and
+// rejects it in a clobber list.  Nothing in these kernels makes the compiler itself keep a value in M0
+// across a statement: no LDS-DMA builtin, no register-indexed moves, accumulators indexed by constants.)
 __device__ __forceinline__ void copy16(const char *base, uint32_t voff, const char *lds_dst) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr(lds_dst)) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr(lds_dst)) : "memory");
 }
 __device__ __forceinline__ void copy4(const char *base, uint32_t voff, const char *lds_dst) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr(lds_dst)) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr(lds_dst)) : "memory");
 }
 // A wave-uniform pointer, read through lane 0 so that the compiler keeps it in scalar registers.
 __device__ __forceinline__ const char *uniform_ptr(const char *p) {

@@ -1,17 +1,21 @@
 #!/usr/bin/env python3
 """Benchmark of the fused-MoE forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME] [--split 0|1] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME] [--split 0|1] [--headline-only]
+    python bench.py --sweep [--sweep-out FILE.csv]
 
 A "step" is one call of the fused op over one batch of synthetic input that is already
 resident in HBM (routing, moe_align and quantisation happen before the timed region, as in the
-reference's benchmark/benchmark.py:19-22).  The default workload is the Mixtral-8x7B-like bf16
+reference's benchmark/benchmark.py:19-22).  The headline workload is the Mixtral-8x7B-like bf16
 prefill shape with split=True.  The last line printed is one JSON object: whole-op throughput
-(`value`), the roofline figure of the dominant kernel measured with HIP events in this run, and
-the CPU oracle timed on the host cores on a bounded sample of the same workload.
+(`value`), the roofline figure of the dominant kernel measured with HIP events in this run, the
+CPU oracle timed on the host cores on a bounded sample of the same workload, and `config.all`: the
+same measurements (time, TFLOP/s, GB/s, % of roofline, per-kernel times) for every benchmark
+configuration and both values of `split` where the specification names both, taken before the
+headline run (`--headline-only` skips them), plus the router front-end next to the unfused sequence.
 
-`--all` additionally prints one line per benchmark configuration (time, TFLOP/s, GB/s, % of
-roofline) to stderr.
+`--sweep` runs the reference benchmark's token sweep against torch's grouped GEMM on this GPU and
+writes a CSV with the reference's columns (prime_moe/sweep.py).
 """
 from __future__ import annotations
 
@@ -104,16 +108,21 @@ def phase_time(step, mask, steps):
         lib.pmoe_set_phase_mask(PHASE_ALL)
 
 
-# L2-miss traffic of the roofline kernel per launch, bytes: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 of two
-# `rocprofv3 --pmc` runs of this script (scale factors from the plain 1 GiB copy of --calibrate-copy);
-# the summaries the figures come from are kept under profiles/.  A counter run cannot share a process
-# with the timed run, so the line reports the recorded figure of the same kernel and workload.
-MEASURED_TRAFFIC = {
-    ("c2_mixtral_bf16", 1): 7.15e9,   # moe_up_kernel<bf16>
-    ("c4_dsv3_mxfp8", 1): 8.38e9,     # moe_up_kernel<mxfp8>
-    ("c5_decode_mxfp8", 1): 3.68e9,   # moe_up_kernel<mxfp8>
-    ("c3_qwen3_bf16", 1): 2.13e9,     # moe_up_kernel<bf16>
-}
+def recorded_traffic(config: str, kernel: str = "moe_up_kernel"):
+    """HBM-side bytes per launch of `kernel` on `config` as the last counter run recorded them in
+    profiles/kernel_figures.txt (written by prime_moe/profiling.py: FETCH_SIZE + WRITE_SIZE of two
+    rocprofv3 --pmc runs, scaled by a plain copy of known size).  A counter run cannot share a process
+    with the timed run, so the line carries the recorded figure and says where it comes from."""
+    path = os.path.join(ROOT, "profiles", "kernel_figures.txt")
+    try:
+        for line in open(path):
+            f = line.split()
+            if len(f) >= 8 and f[0] == config and f[1] == kernel:
+                kv = dict(zip(f[2::2], f[3::2]))
+                return float(kv["fetch_bytes"]) + float(kv["write_bytes"]), float(kv.get("mfma_busy", "nan"))
+    except OSError:
+        pass
+    return None, None
 
 
 def hbm_bytes(cfg, inp):
@@ -229,6 +238,39 @@ def run_config(cfg, split, steps, warmup, device, with_cpu, log):
     return res
 
 
+def router_times(device, steps):
+    """The router front-end (top-k + softmax + moe_align, prime_moe.route) next to the unfused torch
+    sequence in front of the moe_align op, on the gate logits of the Qwen3-like configuration."""
+    import prime_moe
+    from prime_moe.workloads import CONFIGS
+    cfg = CONFIGS["c3_qwen3_bf16"]
+    g = torch.Generator(device=device).manual_seed(0)
+    logits = torch.randn((cfg.T, cfg.E), generator=g, device=device)
+
+    def unfused():
+        vals, ids = torch.topk(logits, cfg.top_k, dim=-1)
+        w = torch.softmax(vals.float(), dim=-1)
+        return (ids.to(torch.int32), w) + tuple(torch.ops.prime_moe.moe_align(ids.to(torch.int32), cfg.E, cfg.block_m, 1))
+
+    fused = lambda: prime_moe.route(logits, cfg.top_k, cfg.block_m, 1)
+    out = {}
+    for name, fn in (("fused_us", fused), ("unfused_us", unfused)):
+        for _ in range(5):
+            fn()
+        out[name] = time_events(fn, steps)[1] * 1e6
+    out["workload"] = f"gate logits ({cfg.T}, {cfg.E}) fp32, top_k={cfg.top_k}, block_m=128"
+    return out
+
+
+def summary(r):
+    """One entry of `config.all`."""
+    return {"config": r["name"], "split": r["split"], "us_per_call": round(r["sec"] * 1e6, 1),
+            "tflops": round(r["tflops"], 1), "pct_mfma_peak": round(r["pct_mfma"], 2),
+            "weight_gbs": round(r["weight_gbs"], 1), "pct_hbm_all_bytes": round(r["pct_hbm"], 2),
+            "up_kernel_us": round(r["t_up"] * 1e6, 1), "down_kernel_us": round(r["t_down"] * 1e6, 1),
+            "other_us": round((r["ev_mean"] - r["t_up"] - r["t_down"]) * 1e6, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -236,11 +278,16 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="c2_mixtral_bf16")
     ap.add_argument("--split", type=int, default=1)
-    ap.add_argument("--all", action="store_true", help="also time every benchmark configuration (stderr)")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="time only --config (skips the other configurations and the router)")
+    ap.add_argument("--all", action="store_true", help="(accepted for compatibility: every configuration is timed by default)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU oracle leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (a kernel of known traffic, to scale the "
-                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run); implies --headline-only")
+    ap.add_argument("--sweep", action="store_true", help="token sweep against torch's grouped GEMM, CSV output")
+    ap.add_argument("--sweep-out", default=os.path.join(ROOT, "gpurun_out", "sweep.csv"))
+    ap.add_argument("--sweep-tokens", type=int, nargs="+", default=[4096, 8192, 16384, 32768, 65536, 131072])
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path is single-device, "
@@ -252,6 +299,13 @@ def main():
     log = lambda *a: print(*a, file=sys.stderr, flush=True)
     log(f"device: {torch.cuda.get_device_name(0)}; peaks used: bf16 {PEAK_TFLOPS['bf16']} / "
         f"mxfp8 {PEAK_TFLOPS['mxfp8']} TFLOP/s dense, HBM {PEAK_HBM_GBS} GB/s")
+    if args.sweep:
+        from prime_moe.sweep import run_sweep
+        os.makedirs(os.path.dirname(os.path.abspath(args.sweep_out)), exist_ok=True)
+        rows = run_sweep(args.sweep_out, tokens=tuple(args.sweep_tokens), warmup=min(args.warmup, 10), iters=args.steps, log=log)
+        print(json.dumps({"sweep_csv": args.sweep_out, "rows": len(rows),
+                          "speedup_min": min(r["speedup"] for r in rows), "speedup_max": max(r["speedup"] for r in rows)}))
+        return
     if args.calibrate_copy:
         from prime_moe import _native
         src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
@@ -262,17 +316,23 @@ def main():
         torch.cuda.synchronize()
         del src, dst
         torch.cuda.empty_cache()
-    if args.all:
+    everything, router = [], None
+    if not (args.headline_only or args.calibrate_copy or args.config != "c2_mixtral_bf16" or args.split != 1):
+        # every configuration, both pipelines where the specification names both; also brings the chip to
+        # its steady clocks before the headline run
         for name, cfg in CONFIGS.items():
-            if name == args.config:
-                continue
-            for split in (1, 0):
-                n_steps = max(5, args.steps // 2)
-                run_config(cfg, split, n_steps, 2, device, False, log)
+            for split in ((1, 0) if name.startswith(("c2", "c5")) else (1,)):
+                if name == args.config and split == args.split:
+                    continue
+                everything.append(summary(run_config(cfg, split, max(5, args.steps // 2), 5, device, False, log)))
                 torch.cuda.empty_cache()
+        router = router_times(device, 20)
+        log(f"router front-end on {router['workload']}: fused {router['fused_us']:.1f} us, "
+            f"torch top-k + softmax + moe_align op {router['unfused_us']:.1f} us")
     cfg = CONFIGS[args.config]
     r = run_config(cfg, args.split, args.steps, args.warmup, device,
                    with_cpu=not args.no_cpu, log=log)
+    everything.insert(0, summary(r))
     memory_bound = cfg.name.startswith("c5")
     if cfg.dtype != "bf16":
         # the mxfp8 shapes stream every touched weight once (arithmetic intensity below the ridge): the up
@@ -290,7 +350,11 @@ def main():
                     "peak": PEAK_TFLOPS[cfg.dtype], "unit": "TFLOP/s",
                     "kernel": "moe_up_kernel (gate/up GEMM + SwiGLU)", "launch_us": r["t_up"] * 1e6}
     roofline["frac"] = roofline["achieved"] / roofline["peak"]
-    roofline["traffic"] = MEASURED_TRAFFIC.get((cfg.name, 1))  # the kernels do not depend on --split
+    traffic, mfma_busy = recorded_traffic(cfg.name)  # the kernels do not depend on --split
+    roofline["traffic"] = traffic
+    roofline["traffic_source"] = ("profiles/kernel_figures.txt (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier run of "
+                                  "this workload, prime_moe/profiling.py)") if traffic is not None else None
+    roofline["mfma_busy_recorded"] = mfma_busy
     line = {
         "metric": "Fused-MoE TFLOP/s & % MFMA peak (bf16/mxfp8); decode-shape HBM GB/s",
         "value": r["weight_gbs"] if memory_bound else r["tflops"],
@@ -301,7 +365,8 @@ def main():
         "config": {"workload": f"{cfg.name}: T={cfg.T} K={cfg.K} E={cfg.E} N={cfg.N} top_k={cfg.top_k} "
                                f"block_m=128 split={bool(args.split)}",
                    "flops_per_step": cfg.flops, "pct_mfma_peak": r["pct_mfma"],
-                   "weight_gbs": r["weight_gbs"], "parity_rel_clamp_1": r["parity"]},
+                   "weight_gbs": r["weight_gbs"], "parity_rel_clamp_1": r["parity"],
+                   "all": everything, "router": router},
         "roofline": roofline,
         "cpu_baseline": r["cpu"],
     }

@@ -97,6 +97,7 @@ __device__ __forceinline__ bool resolve_job(const MoeArgs &a, Job &j) {
 template <int NG>
 struct RowInfo {
     int tok[kBlockRows * NG];   // token index of each sorted row, -1 for padding / dropped rows
+    int pair[kBlockRows * NG];  // its pair id (the row of y it writes), -1 likewise
     int nvalid[NG];             // per group: 1 + index of the last live row
 };
 
@@ -109,16 +110,17 @@ __device__ __forceinline__ int load_row_info(const MoeArgs &a, int first, int nb
     __syncthreads();
     if (tid < kBlockRows * NG) {
         const int g = tid >> 7;
-        int tok = -1;
+        int tok = -1, pair = -1;
         if (g < nb) {
             const int s = first * kBlockRows + tid;
             const int p = (s < a.sorted_num) ? a.sorted_ids[s] : -1;
-            if (p >= 0) {
+            if (p >= 0 && p / a.top_k < a.M) {
                 tok = p / a.top_k;
-                if (tok >= a.M) tok = -1;
+                pair = p;
             }
         }
         ri.tok[tid] = tok;
+        ri.pair[tid] = pair;
         if (tok >= 0) atomicMax(&ri.nvalid[g], (tid & 127) + 1);
     }
     __syncthreads();
@@ -161,17 +163,20 @@ __device__ __forceinline__ void y_epilogue(const f32x16 (&acc)[2][4], char *tile
         }
     }
 }
-// Where a group's 128 x 256 output tile goes: y rows of the sorted order (row pitch K, the last tile of
-// a K that is not a multiple of 256 has 128 columns) or a tile of y_tail (256 x 256, pitch 512 bytes).
+// Where a group's 128 x 256 output tile goes: the y rows of its pairs (y is indexed by pair id, row pitch
+// K; the last tile of a K that is not a multiple of 256 has 128 columns) or a tile of y_tail (256 x 256,
+// pitch 512 bytes).
 struct YDst {
-    char *base;     // first row, first column of the group's tile
+    char *base;     // first column of the group's tile: in row 0 of y (by_pair) or in the tile's first row
     int64_t pitch;  // bytes per row
     int cols;       // columns to write
+    bool by_pair;   // row r of the tile goes to y row pair[r] (else to row r of a y_tail tile)
 };
 __device__ __forceinline__ YDst y_destination(const MoeArgs &a, const Job &j, int grp, int k0) {
     YDst d;
+    d.by_pair = j.part == 0;
     if (j.part == 0) {
-        d.base = a.y + (((int64_t)(j.first + grp) * kBlockRows) * a.K + k0) * 2;
+        d.base = a.y + (int64_t)k0 * 2;
         d.pitch = (int64_t)a.K * 2;
         d.cols = min(kWRows, a.K - k0);
     } else {
@@ -183,10 +188,12 @@ __device__ __forceinline__ YDst y_destination(const MoeArgs &a, const Job &j, in
 }
 // Tiles with a single live fragment skip the detour through LDS: every lane stores its 8-byte runs
 // straight to the destination (32 rows x 16 KB per tile at most; a barrier and an LDS round trip cost more).
-__device__ __forceinline__ void store_y_direct(const YDst &d, const f32x16 (&acc)[2][4], int n_rows, int w4, int lane) {
+// `pair_r` = pair id of this lane's row (lane % 32) of the group, < 0 if the row holds none.
+__device__ __forceinline__ void store_y_direct(const YDst &d, const f32x16 (&acc)[2][4], int n_rows, int w4, int lane,
+                                               int pair_r) {
     const int r = lane & 31, half = lane >> 5;
-    if (r >= n_rows) return;
-    char *dst = d.base + r * d.pitch;
+    if (r >= n_rows || (d.by_pair && pair_r < 0)) return;
+    char *dst = d.base + (d.by_pair ? pair_r : r) * d.pitch;
 #pragma unroll
     for (int f = 0; f < 2; ++f)
 #pragma unroll
@@ -200,16 +207,20 @@ __device__ __forceinline__ void store_y_direct(const YDst &d, const f32x16 (&acc
             }
         }
 }
-// ... and its first n_rows rows are copied to the destination; gt = thread index inside the group.
-__device__ __forceinline__ void store_y_tile(const YDst &d, const char *tile, int n_rows, int gt) {
+// ... and its first n_rows rows are copied to the destination; gt = thread index inside the group,
+// `pair` = the pair ids of the group's 128 rows (rows without one are skipped).
+__device__ __forceinline__ void store_y_tile(const YDst &d, const char *tile, int n_rows, int gt, const int *pair) {
     const int c = gt & 31;
     if (8 * c >= d.cols) return;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int row = (gt >> 5) + 8 * i;
         if (row < n_rows) {
-            const uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kYPitch + c * 16);
-            *reinterpret_cast<uint4 *>(d.base + row * d.pitch + c * 16) = v;
+            const int dst_row = d.by_pair ? pair[row] : row;
+            if (dst_row >= 0) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kYPitch + c * 16);
+                *reinterpret_cast<uint4 *>(d.base + dst_row * d.pitch + c * 16) = v;
+            }
         }
     }
 }
@@ -509,6 +520,9 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, const Job &job, R
 template <int DT>
 struct SplitLds {
     static constexpr int kRowInfoBytes = 2304;  // >= sizeof(RowInfo<2>)
+    // bf16: the pair ids of the tile's rows, fetched again for the down kernel's epilogue (the ring has run
+    // over the row table by then); behind the two output tiles of the epilogue
+    static constexpr int kPairOff = 140 * 1024;
     static constexpr int kRing = DT == DT_BF16 ? ring128::kRingBytes : ring::ring_bytes<DT>();
     static constexpr int kRowInfoOff = DT == DT_BF16 ? kRing - kRowInfoBytes : kRing;
     static constexpr int kActScaleOff = kRowInfoOff + kRowInfoBytes;  // mxfp8 only
@@ -605,6 +619,7 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, const Job &job,
     const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
     const int my_ntf = grp ? ntf1 : ntf0;
     const int my_rows = ri.nvalid[grp];  // rows past the last live one are never read back
+    const int my_pair = ri.pair[grp * kBlockRows + (lane & 31)];  // (tiles of one fragment store from registers)
     const bool active = my_ntf > 0;
     const ring::Layout lay = ring::make_layout<DT, RB>(ntf0, ntf1, ring::ring_bytes<DT>());
 
@@ -661,12 +676,12 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, const Job &job,
         }
         const YDst dst = y_destination(a, job, grp, k0);
         if constexpr (NTF == 1) {
-            if (active) store_y_direct(dst, acc, my_rows, w4, lane);
+            if (active) store_y_direct(dst, acc, my_rows, w4, lane, my_pair);
         } else {
             char *tile = lds + grp * (kBlockRows * kYPitch);
             if (active) y_epilogue<NTF>(acc, tile, w4, lane);
             __syncthreads();
-            if (active) store_y_tile(dst, tile, my_rows, gt);
+            if (active) store_y_tile(dst, tile, my_rows, gt, ri.pair + grp * kBlockRows);
             if (more) __syncthreads();  // the tiles have been read: the head of the ring may be filled again
         }
         k0 += kWRows;
@@ -686,6 +701,7 @@ __device__ __forceinline__ void down_tile_wide_bf16(const MoeArgs &a, const Job 
     const int ntf1 = __builtin_amdgcn_readfirstlane((ri.nvalid[1] + 31) >> 5);
     const int my_ntf = grp ? ntf1 : ntf0;
     const int my_rows = ri.nvalid[grp];  // read before the ring overwrites the row table
+    const int my_pair = ri.pair[grp * kBlockRows + (lane & 31)];
     const bool active = my_ntf > 0;
 
     const uint32_t row_bytes = (uint32_t)H * 2u;
@@ -708,12 +724,18 @@ __device__ __forceinline__ void down_tile_wide_bf16(const MoeArgs &a, const Job 
     else ring128::main_loop<NTF, true, false>(acc, ld, lds, n_slabs, wrow, lane, tok_region, start);
     const YDst dst = y_destination(a, job, grp, k0);
     if constexpr (NTF == 1) {
-        if (active) store_y_direct(dst, acc, my_rows, w4, lane);
+        if (active) store_y_direct(dst, acc, my_rows, w4, lane, my_pair);
     } else {
         char *tile = lds + grp * (kBlockRows * kYPitch);
+        int *pair = reinterpret_cast<int *>(lds + SplitLds<DT_BF16>::kPairOff);
+        if (tid < 2 * kBlockRows) {  // the same test as load_row_info's: a pair id whose token is out of range is none
+            const int64_t srow = row0 + tid;
+            const int p = (tid < job.nb * kBlockRows && srow < a.sorted_num) ? a.sorted_ids[srow] : -1;
+            pair[tid] = (p >= 0 && p / a.top_k < a.M) ? p : -1;
+        }
         if (active) y_epilogue<NTF>(acc, tile, w4, lane);
         __syncthreads();
-        if (active) store_y_tile(dst, tile, my_rows, gt);
+        if (active) store_y_tile(dst, tile, my_rows, gt, pair + grp * kBlockRows);
     }
 }
 
@@ -768,8 +790,9 @@ struct TailSplit {
 };
 
 // How the tail of `n_jobs` jobs on `n_cus` CUs is split: at most `max_jobs` of them, every part gets at
-// least one slab, and the parts > 0 fit the kTailSlots entries behind the list.
-__device__ __forceinline__ void plan_tail_split(TailSplit &ts, int n_jobs, int n_cus, int n_slabs, int max_jobs) {
+// least one slab, and the parts > 0 fit `extra_cap` (<= kTailSlots) entries behind the list.
+__device__ __forceinline__ void plan_tail_split(TailSplit &ts, int n_jobs, int n_cus, int n_slabs, int max_jobs,
+                                                int extra_cap) {
     ts.parts = 1;
     ts.per_xcd_tail = 0;
     if (n_cus <= 0 || n_jobs <= 0) return;
@@ -778,7 +801,7 @@ __device__ __forceinline__ void plan_tail_split(TailSplit &ts, int n_jobs, int n
     int parts = min(min(4, n_slabs), n_cus / rest);
     const int per_xcd_tail = (rest + 7) >> 3;
     if (per_xcd_tail * 8 > max_jobs) return;
-    while (parts > 1 && per_xcd_tail * 8 * (parts - 1) > kTailSlots) --parts;
+    while (parts > 1 && per_xcd_tail * 8 * (parts - 1) > extra_cap) --parts;
     if (parts < 2) return;
     ts.parts = parts;
     ts.per_xcd_tail = per_xcd_tail;
@@ -820,7 +843,8 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
                                                            int4 *work_up, int n_wt_up, int per_job_up, int grid_up,
                                                            int4 *work_down, int n_wt_down, int per_job_down,
                                                            int grid_down, int split_cus, int up_slabs, int down_slabs,
-                                                           int *tail_tab, int *up_counters, int num_experts,
+                                                           int *tail_tab, int *up_counters, int down_tail_tiles,
+                                                           int up_tail_jobs, int num_experts,
                                                            const int32_t *sorted_ids, int sorted_num, int32_t *inv,
                                                            int n_pairs, int do_invert, const uint8_t *x_scales,
                                                            uint32_t *xs_tiled, int nkt, int top_k, int M) {
@@ -877,11 +901,11 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
         ts.extra_base = grid_down - kTailSlots;
         ts.tail_tab = tail_tab;
         plan_tail_split(ts, tail_tab != nullptr ? nt * ((n_wt_down + per_job_down - 1) / per_job_down) : 0, split_cus,
-                        down_slabs, kTailSlots);
+                        down_slabs, down_tail_tiles, down_tail_tiles);
         ts_up.extra_base = grid_up - kTailSlots;
         ts_up.tail_tab = nullptr;
         plan_tail_split(ts_up, up_counters != nullptr ? nt * ((n_wt_up + per_job_up - 1) / per_job_up) : 0, split_cus,
-                        up_slabs, kUpTailJobs);
+                        up_slabs, up_tail_jobs, kTailSlots);
         for (int t = tid; t < nt; t += 256) {
             const int2 tl = tiles[t];
             const int e = expert_ids[tl.x];
@@ -895,7 +919,8 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
         const int stride = (int)(gridDim.x * blockDim.x);
         for (int s = (int)(blockIdx.x * blockDim.x + threadIdx.x); s < n_rows; s += stride) {
             const int p = sorted_ids[s];
-            if (p >= 0 && p < n_pairs) inv[p] = s;
+            const int e = expert_ids[s >> 7];  // rows of a block without an expert are not computed
+            if (p >= 0 && p < n_pairs && e >= 0 && e < num_experts) inv[p] = s;
         }
     }
     if (do_invert && xs_tiled != nullptr) {
@@ -937,15 +962,18 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
     }
 }
 
-// out[t, 8 columns] = bf16(sum over the token's top_k pairs p, in pair order, of w[p] * y[row(p)])
-// (y[row] = the row's part 0 plus, for tiles the down kernel split, the partial rows in y_tail)
-// (ACCUMULATE: added to what `out` holds).  row(p) = inv[p] if that row really holds p, else the
-// pair was dropped by the schedule and contributes nothing.  One thread per (token, 8 columns).
+// out[t, 8 columns] = bf16(sum over the token's top_k pairs p, in pair order, of w[p] * y[p])
+// (y[p] = part 0 of the pair's down projection plus, for tiles the down kernel split, the partial rows in
+// y_tail, found through the pair's sorted row) (ACCUMULATE: added to what `out` holds).  A pair counts if
+// inv[p] is a row of the schedule that really holds p in a block with an expert; otherwise the schedule
+// dropped it, nobody wrote y[p], and it contributes nothing.  A pair id that the schedule lists more than
+// once contributes once.  One thread per (token, 8 columns).
 template <bool ACCUMULATE>
 __global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int32_t *inv, const int32_t *sorted_ids,
                                                        const int32_t *ntpp, int sorted_num, const float *topk_w,
                                                        int top_k, int M, int K, uint4 *out, const int *tail_tab,
-                                                       const char *y_tail, int n_wt) {
+                                                       const char *y_tail, int n_wt, const int32_t *expert_ids,
+                                                       int num_experts) {
     const int k8 = K >> 3;
     const int64_t total = (int64_t)M * k8;
     const int n_rows = min(ntpp[0], sorted_num);
@@ -957,6 +985,8 @@ __global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int3
             const int p = t * top_k + r;
             const int row = inv[p];
             if (row < 0 || row >= n_rows || sorted_ids[row] != p) continue;
+            const int e = expert_ids[row >> 7];
+            if (e < 0 || e >= num_experts) continue;
             const float w = topk_w[p];
             auto add = [&](const uint4 q) {
                 const uint32_t u[4] = {q.x, q.y, q.z, q.w};
@@ -966,7 +996,7 @@ __global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int3
                     v[2 * j + 1] += w * bf16_bits_to_f32(u[j] >> 16);
                 }
             };
-            add(*reinterpret_cast<const uint4 *>(y + ((int64_t)row * K + 8 * c) * 2));
+            add(*reinterpret_cast<const uint4 *>(y + ((int64_t)p * K + 8 * c) * 2));
             // a tile whose contraction was split: the other parts' partial rows, in part order
             const int tt = tail_tab != nullptr ? tail_tab[(row >> 7) * n_wt + (c >> 5)] : 0;
             if (tt != 0) {
@@ -997,6 +1027,7 @@ struct WorkspaceLayout {
     size_t n_tiles_off, up_counters_off, tiles_off, work_up_off, work_down_off, tail_tab_off, y_tail_off,
         up_partials_off, inv_off, y_off, act_off,
         act_scales_off, xs_tiled_off, total;
+    int down_tail_tiles, up_tail_jobs;  // partial tiles y_tail holds / jobs up_partials holds (0: no split tails)
 };
 
 static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_num, int top_k) {
@@ -1018,14 +1049,18 @@ static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_
     off = align_up(off + (align_up(blocks * n_wt_down, 8) + kTailSlots) * sizeof(int4), 256);
     l.tail_tab_off = off;
     if (dt == DT_BF16) off = align_up(off + blocks * n_wt_down * sizeof(int32_t), 256);
+    // split tail jobs: no more of them than there are jobs; up to 3 partial tiles per down job
+    l.down_tail_tiles = dt == DT_BF16 ? (int)std::min<size_t>(kTailSlots, 3 * align_up(blocks * n_wt_down, 8)) : 0;
+    l.up_tail_jobs = dt == DT_BF16 ? (int)std::min<size_t>(kUpTailJobs, align_up(blocks * (H / 128), 8)) : 0;
     l.y_tail_off = off;
-    if (dt == DT_BF16) off = align_up(off + (size_t)kTailSlots * kWRows * kWRows * 2, 256);
+    off = align_up(off + (size_t)l.down_tail_tiles * kWRows * kWRows * 2, 256);
     l.up_partials_off = off;  // 4 parts x 512 threads x 128 floats per job
-    if (dt == DT_BF16) off = align_up(off + (size_t)kUpTailJobs * 4 * 512 * 128 * sizeof(float), 256);
+    off = align_up(off + (size_t)l.up_tail_jobs * 4 * 512 * 128 * sizeof(float), 256);
     l.inv_off = off;
-    off = align_up(off + (size_t)M * (size_t)std::max(top_k, 1) * sizeof(int32_t), 256);
-    l.y_off = off;
-    off = align_up(off + rows * K * 2, 256);
+    const size_t pairs = (size_t)M * (size_t)std::max(top_k, 1);
+    off = align_up(off + pairs * sizeof(int32_t), 256);
+    l.y_off = off;  // one row per pair id
+    off = align_up(off + pairs * K * 2, 256);
     l.act_off = off;
     off = align_up(off + rows * H * (dt == DT_BF16 ? 2 : 1), 256);
     l.act_scales_off = off;
@@ -1079,6 +1114,7 @@ struct SchedBuffers {
     int4 *work_down;
     int *tail_tab;     // null: the down kernel's tail is not split (mxfp8)
     int *up_counters;  // null: the up kernel's tail is not split (mxfp8)
+    int down_tail_tiles, up_tail_jobs;  // capacities of y_tail and up_partials
 };
 
 template <int DT>
@@ -1100,7 +1136,7 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
         hipLaunchKernelGGL(moe_prologue_kernel, dim3(blocks), dim3(256), 0, s, a.expert_ids, a.ntpp, a.n_blocks,
                            sb.tiles, sb.n_tiles, sb.work_up, a.n_wtiles, per_up, grid_up,
                            sb.work_down, n_wt_down, per_down, grid_down, resident_grid(), a.K * 2 / 128, a.H * 2 / 128,
-                           sb.tail_tab, sb.up_counters, a.E,
+                           sb.tail_tab, sb.up_counters, sb.down_tail_tiles, sb.up_tail_jobs, a.E,
                            a.sorted_ids, a.sorted_num, a.inv, a.M * a.top_k, do_invert, a.x_scales, a.xs_tiled,
                            a.K >> 7, a.top_k, a.M);
     }
@@ -1120,11 +1156,11 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
         if (split)
             hipLaunchKernelGGL(finalize_kernel<false>, dim3(blocks), dim3(256), 0, s, a.y, a.inv, a.sorted_ids, a.ntpp,
                                a.sorted_num, a.topk_w, a.top_k, a.M, a.K, reinterpret_cast<uint4 *>(out), sb.tail_tab,
-                               a.y_tail, n_wt_down);
+                               a.y_tail, n_wt_down, a.expert_ids, a.E);
         else
             hipLaunchKernelGGL(finalize_kernel<true>, dim3(blocks), dim3(256), 0, s, a.y, a.inv, a.sorted_ids, a.ntpp,
                                a.sorted_num, a.topk_w, a.top_k, a.M, a.K, reinterpret_cast<uint4 *>(out), sb.tail_tab,
-                               a.y_tail, n_wt_down);
+                               a.y_tail, n_wt_down, a.expert_ids, a.E);
     }
     return check_launch("fused_moe launch");
 }
@@ -1135,8 +1171,10 @@ static SchedBuffers sched_buffers(char *ws, const WorkspaceLayout &l) {
     sb.tiles = reinterpret_cast<int2 *>(ws + l.tiles_off);
     sb.work_up = reinterpret_cast<int4 *>(ws + l.work_up_off);
     sb.work_down = reinterpret_cast<int4 *>(ws + l.work_down_off);
-    sb.tail_tab = l.y_tail_off > l.tail_tab_off ? reinterpret_cast<int *>(ws + l.tail_tab_off) : nullptr;
-    sb.up_counters = sb.tail_tab != nullptr ? reinterpret_cast<int *>(ws + l.up_counters_off) : nullptr;
+    sb.tail_tab = l.down_tail_tiles > 0 ? reinterpret_cast<int *>(ws + l.tail_tab_off) : nullptr;
+    sb.up_counters = l.up_tail_jobs > 0 ? reinterpret_cast<int *>(ws + l.up_counters_off) : nullptr;
+    sb.down_tail_tiles = l.down_tail_tiles;
+    sb.up_tail_jobs = l.up_tail_jobs;
     return sb;
 }
 

@@ -161,3 +161,41 @@ def test_result_is_bitwise_reproducible(device):
         outs.append(out)
     torch.cuda.synchronize()
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
+def test_block_without_expert_and_duplicate_pair(device):
+    """Schedules the fused op must survive: a block whose expert id is out of range is not computed and
+    its pairs contribute nothing (never whatever the workspace held); a pair id listed twice contributes
+    once."""
+    import prime_moe
+    T, K, E, N, top_k = 300, 512, 6, 512, 2
+    g, x, w1, w2 = _inputs(T, K, E, N, device, seed=9)
+    ids, wts = reference_routing(T, E, top_k, device, g, hot_last=False)
+    s, e, n = torch.ops.prime_moe.moe_align(ids, E, 128, 1)
+    dropped = 1  # second block of the schedule loses its expert
+    e_bad = e.clone()
+    e_bad[dropped] = -1
+    pairs = s[dropped * 128:(dropped + 1) * 128]
+    pairs = pairs[pairs >= 0].long()
+    w_ref = wts.clone().flatten()
+    w_ref[pairs] = 0.0  # the oracle drops the same pairs through their routing weights
+    ref = O.fused_moe_dense(x.cpu(), w1.cpu(), w2.cpu(), ids.cpu(), w_ref.view(T, top_k).cpu())
+    for fill in (float("nan"), 1e30):  # whatever an earlier call left in the caching allocator's blocks
+        junk = torch.full((64 << 20,), fill, dtype=torch.bfloat16, device=device)
+        del junk
+        out = torch.empty((T, K), dtype=torch.bfloat16, device=device)
+        prime_moe.fused_moe_bf16(x, w1, w2, s, e_bad, n, wts, out, top_k, 128, 64, 4, 2, 1, 1, True)
+        torch.cuda.synchronize()
+        got = out.float().cpu()
+        assert torch.isfinite(got).all()
+        assert rel_clamp(got, ref, 1.0) <= BF16_GATE
+    # a pair id listed twice (in a padding slot of its own block): counted once
+    s_dup = s.clone()
+    blk = int((s[:128] < 0).nonzero()[0]) if bool((s[:128] < 0).any()) else None
+    if blk is not None:
+        s_dup[blk] = s[0]
+        ref = O.fused_moe_dense(x.cpu(), w1.cpu(), w2.cpu(), ids.cpu(), wts.cpu())
+        out = torch.empty((T, K), dtype=torch.bfloat16, device=device)
+        prime_moe.fused_moe_bf16(x, w1, w2, s_dup, e, n, wts, out, top_k, 128, 64, 4, 2, 1, 1, True)
+        torch.cuda.synchronize()
+        assert rel_clamp(out.float().cpu(), ref, 1.0) <= BF16_GATE

@@ -968,12 +968,13 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
 // inv[p] is a row of the schedule that really holds p in a block with an expert; otherwise the schedule
 // dropped it, nobody wrote y[p], and it contributes nothing.  A pair id that the schedule lists more than
 // once contributes once.  One thread per (token, 8 columns).
-template <bool ACCUMULATE>
+template <bool ACCUMULATE, int G>
 __global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int32_t *inv, const int32_t *sorted_ids,
                                                        const int32_t *ntpp, int sorted_num, const float *topk_w,
                                                        int top_k, int M, int K, uint4 *out, const int *tail_tab,
                                                        const char *y_tail, int n_wt, const int32_t *expert_ids,
                                                        int num_experts) {
+    // G pairs are resolved and fetched together: their loads are in flight at the same time
     const int k8 = K >> 3;
     const int64_t total = (int64_t)M * k8;
     const int n_rows = min(ntpp[0], sorted_num);
@@ -981,28 +982,53 @@ __global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int3
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
         const int t = (int)(i / k8), c = (int)(i - (int64_t)t * k8);
         float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int r = 0; r < top_k; ++r) {
-            const int p = t * top_k + r;
-            const int row = inv[p];
-            if (row < 0 || row >= n_rows || sorted_ids[row] != p) continue;
-            const int e = expert_ids[row >> 7];
-            if (e < 0 || e >= num_experts) continue;
-            const float w = topk_w[p];
-            auto add = [&](const uint4 q) {
-                const uint32_t u[4] = {q.x, q.y, q.z, q.w};
+        auto add = [&](const uint4 q, float w) {
+            const uint32_t u[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    v[2 * j] += w * bf16_bits_to_f32(u[j] & 0xffffu);
-                    v[2 * j + 1] += w * bf16_bits_to_f32(u[j] >> 16);
+            for (int j = 0; j < 4; ++j) {
+                v[2 * j] += w * bf16_bits_to_f32(u[j] & 0xffffu);
+                v[2 * j + 1] += w * bf16_bits_to_f32(u[j] >> 16);
+            }
+        };
+        for (int r0 = 0; r0 < top_k; r0 += G) {
+            int row[G];
+            float w[G];
+            uint4 q[G];
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const int p = t * top_k + r0 + g;
+                row[g] = r0 + g < top_k ? inv[p] : -1;
+            }
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const int p = t * top_k + r0 + g;
+                bool ok = row[g] >= 0 && row[g] < n_rows;
+                if (ok) ok = sorted_ids[row[g]] == p;
+                if (ok) {
+                    const int e = expert_ids[row[g] >> 7];
+                    ok = e >= 0 && e < num_experts;
                 }
-            };
-            add(*reinterpret_cast<const uint4 *>(y + ((int64_t)p * K + 8 * c) * 2));
-            // a tile whose contraction was split: the other parts' partial rows, in part order
-            const int tt = tail_tab != nullptr ? tail_tab[(row >> 7) * n_wt + (c >> 5)] : 0;
-            if (tt != 0) {
-                const int parts = tt & 15, rr = ((tt >> 4) & 15) * kBlockRows + (row & 127), slot = tt >> 8;
-                for (int part = 1; part < parts; ++part)
-                    add(*reinterpret_cast<const uint4 *>(y_tail + (((int64_t)(slot + part - 1) * 256 + rr) * 256 + 8 * (c & 31)) * 2));
+                if (!ok) row[g] = -1;
+            }
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const int p = t * top_k + r0 + g;
+                if (row[g] >= 0) {
+                    w[g] = topk_w[p];
+                    q[g] = *reinterpret_cast<const uint4 *>(y + ((int64_t)p * K + 8 * c) * 2);
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                if (row[g] < 0) continue;
+                add(q[g], w[g]);
+                // a tile whose contraction was split: the other parts' partial rows, in part order
+                const int tt = tail_tab != nullptr ? tail_tab[(row[g] >> 7) * n_wt + (c >> 5)] : 0;
+                if (tt != 0) {
+                    const int parts = tt & 15, rr = ((tt >> 4) & 15) * kBlockRows + (row[g] & 127), slot = tt >> 8;
+                    for (int part = 1; part < parts; ++part)
+                        add(*reinterpret_cast<const uint4 *>(y_tail + (((int64_t)(slot + part - 1) * 256 + rr) * 256 + 8 * (c & 31)) * 2), w[g]);
+                }
             }
         }
         uint32_t o[4];
@@ -1153,14 +1179,20 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
     if (mask & PMOE_PHASE_FINALIZE) {
         const int64_t n8 = n_out / 8;
         const int blocks = (int)std::min<int64_t>((n8 + 255) / 256, 8192);
-        if (split)
-            hipLaunchKernelGGL(finalize_kernel<false>, dim3(blocks), dim3(256), 0, s, a.y, a.inv, a.sorted_ids, a.ntpp,
-                               a.sorted_num, a.topk_w, a.top_k, a.M, a.K, reinterpret_cast<uint4 *>(out), sb.tail_tab,
-                               a.y_tail, n_wt_down, a.expert_ids, a.E);
-        else
-            hipLaunchKernelGGL(finalize_kernel<true>, dim3(blocks), dim3(256), 0, s, a.y, a.inv, a.sorted_ids, a.ntpp,
-                               a.sorted_num, a.topk_w, a.top_k, a.M, a.K, reinterpret_cast<uint4 *>(out), sb.tail_tab,
-                               a.y_tail, n_wt_down, a.expert_ids, a.E);
+        auto launch = [&](auto kernel) {
+            hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, s, a.y, a.inv, a.sorted_ids, a.ntpp, a.sorted_num,
+                               a.topk_w, a.top_k, a.M, a.K, reinterpret_cast<uint4 *>(out), sb.tail_tab, a.y_tail,
+                               n_wt_down, a.expert_ids, a.E);
+        };
+        if (split) {
+            if (a.top_k <= 2) launch(finalize_kernel<false, 2>);
+            else if (a.top_k <= 4) launch(finalize_kernel<false, 4>);
+            else launch(finalize_kernel<false, 8>);
+        } else {
+            if (a.top_k <= 2) launch(finalize_kernel<true, 2>);
+            else if (a.top_k <= 4) launch(finalize_kernel<true, 4>);
+            else launch(finalize_kernel<true, 8>);
+        }
     }
     return check_launch("fused_moe launch");
 }

@@ -229,6 +229,15 @@ def run_config(cfg, split, steps, warmup, device, with_cpu, log):
         f"({res['pct_mfma']:5.1f}% {cfg.dtype} MFMA peak)  weights {res['weight_gbs']:7.1f} GB/s  "
         f"all-bytes {res['pct_hbm']:5.1f}% of 8 TB/s | up {t_up * 1e6:9.1f} us ({res['up_tflops']:7.1f} TF) "
         f"down {t_down * 1e6:9.1f} us ({res['down_tflops']:7.1f} TF)")
+    # algorithmic bytes of one launch of each kernel: weights (+ scales) of the touched experts once, the routed
+    # rows of the token-side operand once, the output written once
+    sx = 2 if cfg.dtype == "bf16" else 33 / 32
+    n_touched = wb / cfg.weight_bytes_per_expert()
+    alg = {"moe_up_kernel": n_touched * cfg.N * cfg.K * sx + P * cfg.K * sx + P * cfg.H * sx,
+           "moe_down_kernel": n_touched * cfg.K * cfg.H * sx + P * cfg.H * sx + P * cfg.K * 2,
+           "finalize_kernel": P * cfg.K * 2 + cfg.T * cfg.K * 2}
+    res["algorithmic_bytes"] = alg
+    log("  algorithmic bytes per launch: " + " ".join(f"{k} {v:.0f}" for k, v in alg.items()))
     cpu, err = (None, None)
     if with_cpu:
         cpu, err = cpu_baseline(cfg, inp, out, budget_tokens=4096)

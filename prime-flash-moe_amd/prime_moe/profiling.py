@@ -52,8 +52,14 @@ def run_pass(tag, prof_args, bench_args, workdir, log):
     res = subprocess.run(["timeout", "-s", "KILL", "240", *cmd], cwd="/tmp", env=env, capture_output=True, text=True)
     if res.returncode != 0:
         sys.exit(f"profiler pass {tag} failed (rc {res.returncode}):\n{res.stdout[-2000:]}\n{res.stderr[-2000:]}")
-    bench_line = [l for l in res.stderr.splitlines() + res.stdout.splitlines() if l[:2] in ("c1", "c2", "c3", "c4", "c5")]
-    return out_dir, (bench_line[-1] if bench_line else "")
+    lines = res.stderr.splitlines() + res.stdout.splitlines()
+    bench_line = [l for l in lines if l[:2] in ("c1", "c2", "c3", "c4", "c5")]
+    alg = [l for l in lines if "algorithmic bytes per launch:" in l]
+    algorithmic = {}
+    if alg:
+        f = alg[-1].split(":", 1)[1].split()
+        algorithmic = {f[i]: float(f[i + 1]) for i in range(0, len(f) - 1, 2)}
+    return out_dir, (bench_line[-1] if bench_line else ""), algorithmic
 
 
 def kernel_stats(out_dir):
@@ -102,13 +108,13 @@ def main():
     sq = [c.replace("{DT}", "BF16" if dt == "bf16" else "F8") for c in SQ_COUNTERS]
     common = ["--no-cpu", "--headline-only", "--config", a.config, "--split", str(a.split)]
     cmds = []
-    d_stats, bench_line = run_pass("stats", ["--kernel-trace", "--stats"], ["--steps", "10", "--warmup", "3", *common],
+    d_stats, bench_line, algorithmic = run_pass("stats", ["--kernel-trace", "--stats"], ["--steps", "10", "--warmup", "3", *common],
                                    a.workdir, cmds)
-    d_fetch, _ = run_pass("fetch", ["--pmc", "FETCH_SIZE"], ["--steps", "3", "--warmup", "1", "--calibrate-copy", *common],
+    d_fetch, _, _ = run_pass("fetch", ["--pmc", "FETCH_SIZE"], ["--steps", "3", "--warmup", "1", "--calibrate-copy", *common],
                           a.workdir, cmds)
-    d_write, _ = run_pass("write", ["--pmc", "WRITE_SIZE"], ["--steps", "3", "--warmup", "1", "--calibrate-copy", *common],
+    d_write, _, _ = run_pass("write", ["--pmc", "WRITE_SIZE"], ["--steps", "3", "--warmup", "1", "--calibrate-copy", *common],
                           a.workdir, cmds)
-    d_sq, _ = run_pass("sq", ["--pmc", *sq], ["--steps", "3", "--warmup", "1", *common], a.workdir, cmds)
+    d_sq, _, _ = run_pass("sq", ["--pmc", *sq], ["--steps", "3", "--warmup", "1", *common], a.workdir, cmds)
     stats, fetch, write, sqc = kernel_stats(d_stats), counters(d_fetch), counters(d_write), counters(d_sq)
     cal_f = fetch.get("copy_calibration_kernel", {}).get("FETCH_SIZE", (GIB_KIB, 0))[0]
     cal_w = write.get("copy_calibration_kernel", {}).get("WRITE_SIZE", (GIB_KIB, 0))[0]
@@ -124,8 +130,8 @@ def main():
               f"FETCH_SIZE reads {cal_f:,.0f} KiB for it (scale factor {f_scale:.2f}), WRITE_SIZE {cal_w:,.0f} KiB (scale factor {w_scale:.2f}).",
               "", "bench.py's own line of the traced run (profiler attached):", "", "    " + bench_line, "",
               "## Per kernel (means per dispatch)", "",
-              "| kernel | avg duration | fetched past L2 | written past L2 | sum | rate | MFMA busy | LDS conflict cycles / LDS active | waiting on LDS |",
-              "|---|---|---|---|---|---|---|---|---|"]
+              "| kernel | avg duration | fetched past L2 | written past L2 | sum | algorithmic bytes | rate | MFMA busy | LDS conflict cycles / LDS active | waiting on LDS |",
+              "|---|---|---|---|---|---|---|---|---|---|"]
     figs = []
     for k in KERNELS[:4]:
         if k not in stats:
@@ -142,13 +148,15 @@ def main():
         conflict = c.get("SQ_LDS_BANK_CONFLICT", 0.0) / lds_act if lds_act else 0.0
         wait_lds = c.get("SQ_WAIT_INST_LDS", 0.0) / c["SQ_WAVE_CYCLES"] if c.get("SQ_WAVE_CYCLES") else 0.0
         mfma_frac = mfma / busy if busy else 0.0
+        ab = algorithmic.get(k)
         lines.append(f"| {k} | {us:.1f} us | {fb / 1e9:.3f} GB | {wb / 1e9:.3f} GB | {(fb + wb) / 1e9:.3f} GB | "
-                     f"{(fb + wb) / us / 1e6:.2f} TB/s | {mfma_frac:.3f} | {conflict:.3f} | {wait_lds:.3f} |")
+                     f"{(f'{ab / 1e9:.3f} GB' if ab else '')} | {(fb + wb) / us / 1e6:.2f} TB/s | {mfma_frac:.3f} | {conflict:.3f} | {wait_lds:.3f} |")
         figs.append(f"{a.config} {k} avg_us {us:.1f} fetch_bytes {fb:.0f} write_bytes {wb:.0f} mfma_busy {mfma_frac:.4f} "
                     f"lds_conflict {conflict:.4f}")
     lines += ["", "MFMA busy = SQ_VALU_MFMA_BUSY_CYCLES (summed over SIMDs) / (SQ_BUSY_CYCLES (summed over shader engines) x SIMDs per",
               f"shader engine = {simds_per_se:.0f}): the share of the cycles a SIMD is busy in which its matrix pipe is.",
-              "FETCH_SIZE counts what misses the per-XCD L2s, whether the memory-side cache or HBM serves it.", "",
+              "FETCH_SIZE counts what misses the per-XCD L2s, whether the memory-side cache or HBM serves it.  Algorithmic bytes:",
+              "weights (+ scales) of the touched experts once, the routed rows of the token-side operand once, the output once.", "",
               "## Raw figures", ""]
     for k in KERNELS:
         if k in stats:

@@ -49,6 +49,9 @@ struct MoeArgs {
     char *y_tail;         // partial tiles of down jobs whose contraction is split (see plan_tail_split)
     float *up_partials;   // fp32 partial accumulators of up jobs whose contraction is split
     int *up_counters;     // per such job: parts that have stored theirs (zeroed by the prologue)
+    int4 *join_tab;       // per such job, when a separate kernel joins the parts: its tile (see moe_up_join_kernel)
+    int up_part_stride;   // partial accumulators reserved per job (the largest number of parts)
+    int deep_join;        // the parts of split up jobs only store; moe_up_join_kernel adds them and finishes the tiles
     int top_k, M, K, N, H, E, sorted_num;
     int n_blocks;  // sorted_num / 128 (rounded up)
     int n_wtiles;  // weight tiles along the free dimension: H/128 (up) or ceil(K/256) (down)
@@ -309,11 +312,16 @@ __device__ __forceinline__ void store_act_tile(const MoeArgs &a, const char *til
 // from memory: the same bits whichever part is last) and returns true.  Nobody waits for anybody.
 // `lds_flag` is a word of LDS no copy is in flight to.
 constexpr int kUpTailJobs = 64;
+// Few jobs on many CUs (a.deep_join): the contraction is split further (up to kDeepParts parts) and nobody
+// joins here; every part stores and leaves (returns false), and moe_up_join_kernel, with one workgroup per
+// 32 x 128 piece of every tile, adds the parts and runs the epilogue: the join then costs a few microseconds
+// whatever the number of parts, where the last part alone would read parts x 256 KB.
+constexpr int kDeepParts = 8;  // (6 to 8 measure alike on the README shape, 12 and 16 slower: shorter walks, more to join)
 template <int NTF>
 __device__ __forceinline__ bool join_parts(const MoeArgs &a, const Job &j, f32x16 (&acc)[2][4], bool active,
                                            int *lds_flag) {
     const int tid = threadIdx.x;
-    float4 *mine = reinterpret_cast<float4 *>(a.up_partials) + ((int64_t)(j.slot * 4 + j.part) * 32) * 512;
+    float4 *mine = reinterpret_cast<float4 *>(a.up_partials) + ((int64_t)(j.slot * a.up_part_stride + j.part) * 32) * 512;
     if (active) {
 #pragma unroll
         for (int f = 0; f < 2; ++f)
@@ -324,6 +332,7 @@ __device__ __forceinline__ bool join_parts(const MoeArgs &a, const Job &j, f32x1
                     mine[((f * 4 + t) * 4 + q) * 512 + tid] =
                         make_float4(acc[f][t][4 * q], acc[f][t][4 * q + 1], acc[f][t][4 * q + 2], acc[f][t][4 * q + 3]);
     }
+    if (a.deep_join) return false;  // (the kernel boundary orders the stores before the join kernel's loads)
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // the stores above are visible device-wide before the count below
     __syncthreads();
     if (tid == 0) *lds_flag = atomicAdd(&a.up_counters[j.slot], 1);
@@ -334,7 +343,7 @@ __device__ __forceinline__ bool join_parts(const MoeArgs &a, const Job &j, f32x1
     if (active) {
         zero_acc(acc);
         for (int p = 0; p < j.parts; ++p) {
-            const float4 *src = reinterpret_cast<const float4 *>(a.up_partials) + ((int64_t)(j.slot * 4 + p) * 32) * 512;
+            const float4 *src = reinterpret_cast<const float4 *>(a.up_partials) + ((int64_t)(j.slot * a.up_part_stride + p) * 32) * 512;
 #pragma unroll
             for (int f = 0; f < 2; ++f)
 #pragma unroll
@@ -764,6 +773,60 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
     }
 }
 
+// Joins the parts of split up tiles when the up kernel left them in memory (a.deep_join).  One workgroup of
+// 4 waves per (job, row block of the tile, 32-row fragment): thread (w4, lane) takes over what thread
+// (block, w4, lane) of an up workgroup holds for that fragment, 16 gate and 16 up sums, adds the parts in
+// part order, applies SwiGLU and writes its 4 x 4 activation values.  Same sums in the same order as
+// join_parts, so the same bits.
+__global__ __launch_bounds__(256) void moe_up_join_kernel(MoeArgs a) {
+    const int slot = blockIdx.x >> 3, grp = (blockIdx.x >> 2) & 1, t = blockIdx.x & 3;
+    const int4 jt = a.join_tab[slot];
+    const int parts = jt.z;
+    if (parts < 2) return;
+    const int first = jt.x & 0x0fffffff, nb = jt.x >> 28, ht = jt.y & 0xffff;
+    if (grp >= nb) return;
+    const int tid = threadIdx.x, lane = tid & 63, w4 = tid >> 6;
+    const int r = lane & 31, half = lane >> 5;
+    // a fragment without a live row has nothing to write (every wave looks at the same 32 rows)
+    const int64_t srow0 = (int64_t)(first + grp) * kBlockRows + 32 * t;
+    {
+        const int64_t s = srow0 + r;
+        const int p = s < a.sorted_num ? a.sorted_ids[s] : -1;
+        if (__ballot(p >= 0 && p / a.top_k < a.M) == 0) return;
+    }
+    const int src_tid = grp * 256 + tid;
+    float g[16], u[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) g[i] = u[i] = 0.f;
+    const float4 *base = reinterpret_cast<const float4 *>(a.up_partials);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        float4 vg[kDeepParts], vu[kDeepParts];
+#pragma unroll
+        for (int p = 0; p < kDeepParts; ++p)
+            if (p < parts) {
+                const float4 *src = base + ((int64_t)(slot * a.up_part_stride + p) * 32) * 512;
+                vg[p] = src[((0 * 4 + t) * 4 + q) * 512 + src_tid];
+                vu[p] = src[((1 * 4 + t) * 4 + q) * 512 + src_tid];
+            }
+#pragma unroll
+        for (int p = 0; p < kDeepParts; ++p)
+            if (p < parts) {
+                g[4 * q] += vg[p].x; g[4 * q + 1] += vg[p].y; g[4 * q + 2] += vg[p].z; g[4 * q + 3] += vg[p].w;
+                u[4 * q] += vu[p].x; u[4 * q + 1] += vu[p].y; u[4 * q + 2] += vu[p].z; u[4 * q + 3] += vu[p].w;
+            }
+    }
+    char *dst = a.act + ((srow0 + r) * a.H + ht * 128) * 2;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int hl = 32 * w4 + 8 * q + 4 * half;  // tile-local activation column, as in swiglu_epilogue
+        uint2 pk;
+        pk.x = pack2_bf16(swiglu(g[4 * q], u[4 * q]), swiglu(g[4 * q + 1], u[4 * q + 1]));
+        pk.y = pack2_bf16(swiglu(g[4 * q + 2], u[4 * q + 2]), swiglu(g[4 * q + 3], u[4 * q + 3]));
+        *reinterpret_cast<uint2 *>(dst + hl * 2) = pk;
+    }
+}
+
 // Walk order of the tiles of one kernel: [group of 8 weight tiles][row tile][weight tile in group].
 // The ~32 workgroups that run side by side on an XCD are then 4 consecutive row tiles (mostly of one
 // expert) x 8 weight tiles: every token slab they fetch is shared by 8 weight tiles and every weight
@@ -787,18 +850,19 @@ struct TailSplit {
     int per_xcd_tail;  // jobs split at the end of each XCD's range
     int extra_base;    // first work list entry of the parts > 0
     int *tail_tab;     // down kernel: per (block, weight tile) 0, or first y_tail tile << 8 | block inside its tile << 4 | parts
+    int4 *join_tab;    // up kernel with a separate join: per tail job its tile (first block | blocks << 28, weight tile, parts)
 };
 
 // How the tail of `n_jobs` jobs on `n_cus` CUs is split: at most `max_jobs` of them, every part gets at
 // least one slab, and the parts > 0 fit `extra_cap` (<= kTailSlots) entries behind the list.
 __device__ __forceinline__ void plan_tail_split(TailSplit &ts, int n_jobs, int n_cus, int n_slabs, int max_jobs,
-                                                int extra_cap) {
+                                                int extra_cap, int max_parts = 4) {
     ts.parts = 1;
     ts.per_xcd_tail = 0;
     if (n_cus <= 0 || n_jobs <= 0) return;
     const int rounds = n_jobs / n_cus, rest = n_jobs % n_cus;
     if (rest == 0 || rounds >= 16) return;  // nothing left over, or too little to matter
-    int parts = min(min(4, n_slabs), n_cus / rest);
+    int parts = min(min(max_parts, n_slabs), n_cus / rest);
     const int per_xcd_tail = (rest + 7) >> 3;
     if (per_xcd_tail * 8 > max_jobs) return;
     while (parts > 1 && per_xcd_tail * 8 * (parts - 1) > extra_cap) --parts;
@@ -825,6 +889,7 @@ __device__ __forceinline__ void emit_work(int4 *work, int n_wt, int per_job, int
             const int extra = slot * (ts->parts - 1);
             work[8 * pos + xcd] = make_int4(x, y, z, 0);
             for (int p = 1; p < ts->parts; ++p) work[ts->extra_base + extra + p - 1] = make_int4(x, y, z | p, 0);
+            if (ts->join_tab != nullptr) ts->join_tab[slot] = make_int4(x, wt, ts->parts, 0);
             if (ts->tail_tab != nullptr)
                 for (int b = 0; b < nb; ++b) ts->tail_tab[(first + b) * n_wt + wt] = (extra << 8) | (b << 4) | ts->parts;
         } else {
@@ -844,7 +909,8 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
                                                            int4 *work_down, int n_wt_down, int per_job_down,
                                                            int grid_down, int split_cus, int up_slabs, int down_slabs,
                                                            int *tail_tab, int *up_counters, int down_tail_tiles,
-                                                           int up_tail_jobs, int num_experts,
+                                                           int up_tail_jobs, int4 *join_tab, int up_max_parts,
+                                                           int num_experts,
                                                            const int32_t *sorted_ids, int sorted_num, int32_t *inv,
                                                            int n_pairs, int do_invert, const uint8_t *x_scales,
                                                            uint32_t *xs_tiled, int nkt, int top_k, int M) {
@@ -856,6 +922,7 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
         if (tail_tab != nullptr)
             for (int i = tid; i < n_blocks * n_wt_down; i += 256) tail_tab[i] = 0;
         if (up_counters != nullptr && tid < kUpTailJobs) up_counters[tid] = 0;
+        if (join_tab != nullptr && tid < kUpTailJobs) join_tab[tid] = make_int4(0, 0, 0, 0);
         const int n_live = min((ntpp[0] + kBlockRows - 1) / kBlockRows, n_blocks);
         if (tid == 0) { s_carry[0] = 0; s_carry[1] = 0; }
         __syncthreads();
@@ -900,12 +967,14 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
         TailSplit ts, ts_up;
         ts.extra_base = grid_down - kTailSlots;
         ts.tail_tab = tail_tab;
+        ts.join_tab = nullptr;
         plan_tail_split(ts, tail_tab != nullptr ? nt * ((n_wt_down + per_job_down - 1) / per_job_down) : 0, split_cus,
                         down_slabs, down_tail_tiles, down_tail_tiles);
         ts_up.extra_base = grid_up - kTailSlots;
         ts_up.tail_tab = nullptr;
+        ts_up.join_tab = join_tab;
         plan_tail_split(ts_up, up_counters != nullptr ? nt * ((n_wt_up + per_job_up - 1) / per_job_up) : 0, split_cus,
-                        up_slabs, up_tail_jobs, kTailSlots);
+                        up_slabs, up_tail_jobs, kTailSlots, up_max_parts);
         for (int t = tid; t < nt; t += 256) {
             const int2 tl = tiles[t];
             const int e = expert_ids[tl.x];
@@ -1050,10 +1119,12 @@ __global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int3
 // ------------------------------------------------------------------------------------------ host
 
 struct WorkspaceLayout {
-    size_t n_tiles_off, up_counters_off, tiles_off, work_up_off, work_down_off, tail_tab_off, y_tail_off,
+    size_t n_tiles_off, up_counters_off, join_tab_off, tiles_off, work_up_off, work_down_off, tail_tab_off, y_tail_off,
         up_partials_off, inv_off, y_off, act_off,
         act_scales_off, xs_tiled_off, total;
     int down_tail_tiles, up_tail_jobs;  // partial tiles y_tail holds / jobs up_partials holds (0: no split tails)
+    int up_part_stride;                 // partial accumulators per up job: 4, or kDeepParts with the separate join
+    bool deep_join;
 };
 
 static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_num, int top_k) {
@@ -1066,6 +1137,8 @@ static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_
     off += 256;
     l.up_counters_off = off;
     off += kUpTailJobs * sizeof(int32_t);
+    l.join_tab_off = off;
+    off += kUpTailJobs * sizeof(int4);
     l.tiles_off = off;
     off = align_up(off + blocks * sizeof(int2), 256);
     l.work_up_off = off;
@@ -1080,8 +1153,13 @@ static WorkspaceLayout workspace_layout(int dt, int M, int K, int N, int sorted_
     l.up_tail_jobs = dt == DT_BF16 ? (int)std::min<size_t>(kUpTailJobs, align_up(blocks * (H / 128), 8)) : 0;
     l.y_tail_off = off;
     off = align_up(off + (size_t)l.down_tail_tiles * kWRows * kWRows * 2, 256);
-    l.up_partials_off = off;  // 4 parts x 512 threads x 128 floats per job
-    off = align_up(off + (size_t)l.up_tail_jobs * 4 * 512 * 128 * sizeof(float), 256);
+    // few up jobs for the chip (no more than the split can hold) and a contraction long enough to share among
+    // more workgroups: deeper split, joined by a kernel of its own (see moe_up_join_kernel)
+    // (at most kUpTailJobs / 2 jobs, so that the partial sums stay within what the shallow split reserves)
+    l.deep_join = dt == DT_BF16 && blocks * (H / 128) <= (size_t)kUpTailJobs / 2 && K >= 2048;
+    l.up_part_stride = l.deep_join ? kDeepParts : 4;
+    l.up_partials_off = off;  // parts x 512 threads x 128 floats per job
+    off = align_up(off + (size_t)l.up_tail_jobs * l.up_part_stride * 512 * 128 * sizeof(float), 256);
     l.inv_off = off;
     const size_t pairs = (size_t)M * (size_t)std::max(top_k, 1);
     off = align_up(off + pairs * sizeof(int32_t), 256);
@@ -1141,6 +1219,7 @@ struct SchedBuffers {
     int *tail_tab;     // null: the down kernel's tail is not split (mxfp8)
     int *up_counters;  // null: the up kernel's tail is not split (mxfp8)
     int down_tail_tiles, up_tail_jobs;  // capacities of y_tail and up_partials
+    int4 *join_tab;    // null unless the split up jobs are joined by moe_up_join_kernel
 };
 
 template <int DT>
@@ -1162,14 +1241,17 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
         hipLaunchKernelGGL(moe_prologue_kernel, dim3(blocks), dim3(256), 0, s, a.expert_ids, a.ntpp, a.n_blocks,
                            sb.tiles, sb.n_tiles, sb.work_up, a.n_wtiles, per_up, grid_up,
                            sb.work_down, n_wt_down, per_down, grid_down, resident_grid(), a.K * 2 / 128, a.H * 2 / 128,
-                           sb.tail_tab, sb.up_counters, sb.down_tail_tiles, sb.up_tail_jobs, a.E,
+                           sb.tail_tab, sb.up_counters, sb.down_tail_tiles, sb.up_tail_jobs, sb.join_tab,
+                           sb.join_tab != nullptr ? std::min(kDeepParts, std::max(1, a.K * 2 / 128 / 4)) : 4, a.E,
                            a.sorted_ids, a.sorted_num, a.inv, a.M * a.top_k, do_invert, a.x_scales, a.xs_tiled,
                            a.K >> 7, a.top_k, a.M);
     }
     if (a.n_blocks > 0) {
         a.work = sb.work_up;
-        if (mask & PMOE_PHASE_UP)
+        if (mask & PMOE_PHASE_UP) {
             hipLaunchKernelGGL((moe_up_kernel<DT>), dim3(grid_up), dim3(512), 0, s, a);
+            if (a.deep_join) hipLaunchKernelGGL(moe_up_join_kernel, dim3(sb.up_tail_jobs * 8), dim3(256), 0, s, a);
+        }
         MoeArgs d = a;
         d.n_wtiles = n_wt_down;
         d.work = sb.work_down;
@@ -1207,6 +1289,7 @@ static SchedBuffers sched_buffers(char *ws, const WorkspaceLayout &l) {
     sb.up_counters = l.up_tail_jobs > 0 ? reinterpret_cast<int *>(ws + l.up_counters_off) : nullptr;
     sb.down_tail_tiles = l.down_tail_tiles;
     sb.up_tail_jobs = l.up_tail_jobs;
+    sb.join_tab = l.deep_join ? reinterpret_cast<int4 *>(ws + l.join_tab_off) : nullptr;
     return sb;
 }
 
@@ -1274,6 +1357,9 @@ extern "C" int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2,
     a.y_tail = ws + l.y_tail_off;
     a.up_partials = reinterpret_cast<float *>(ws + l.up_partials_off);
     a.up_counters = reinterpret_cast<int *>(ws + l.up_counters_off);
+    a.join_tab = reinterpret_cast<int4 *>(ws + l.join_tab_off);
+    a.up_part_stride = l.up_part_stride;
+    a.deep_join = l.deep_join ? 1 : 0;
     a.inv = reinterpret_cast<int32_t *>(ws + l.inv_off);
     a.act = ws + l.act_off;
     a.top_k = top_k; a.M = M; a.K = K; a.N = N; a.H = N / 2; a.E = num_experts; a.sorted_num = sorted_num;

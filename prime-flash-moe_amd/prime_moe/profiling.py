@@ -29,7 +29,8 @@ import subprocess
 import sys
 
 ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-KERNELS = ("moe_up_kernel", "moe_down_kernel", "finalize_kernel", "moe_prologue_kernel", "copy_calibration_kernel")
+KERNELS = ("moe_up_kernel", "moe_up_join_kernel", "moe_down_kernel", "finalize_kernel", "moe_prologue_kernel",
+           "copy_calibration_kernel")
 SQ_COUNTERS = ["SQ_BUSY_CYCLES", "SQ_VALU_MFMA_BUSY_CYCLES", "SQ_INSTS_VALU_MFMA_MOPS_{DT}", "SQ_LDS_BANK_CONFLICT",
                "SQ_ACTIVE_INST_LDS", "SQ_WAIT_INST_LDS", "SQ_WAVE_CYCLES", "SQ_WAIT_ANY"]
 GIB_KIB = 1048576.0
@@ -133,7 +134,7 @@ def main():
               "| kernel | avg duration | fetched past L2 | written past L2 | sum | algorithmic bytes | rate | MFMA busy | LDS conflict cycles / LDS active | waiting on LDS |",
               "|---|---|---|---|---|---|---|---|---|---|"]
     figs = []
-    for k in KERNELS[:4]:
+    for k in KERNELS[:5]:
         if k not in stats:
             continue
         us = stats[k]["avg_ns"] / 1e3

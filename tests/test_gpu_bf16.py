@@ -199,3 +199,30 @@ def test_block_without_expert_and_duplicate_pair(device):
         prime_moe.fused_moe_bf16(x, w1, w2, s_dup, e, n, wts, out, top_k, 128, 64, 4, 2, 1, 1, True)
         torch.cuda.synchronize()
         assert rel_clamp(out.float().cpu(), ref, 1.0) <= BF16_GATE
+
+
+@pytest.mark.parametrize("T,K,E,N,top_k,exact", [
+    (256, 4096, 8, 512, 4, False),   # the README shape: 8 - 16 row tiles x 2 weight tiles, every tile split 8 ways
+    (40, 2048, 4, 256, 2, False),    # one weight tile, tiles of one or two fragments
+    (130, 6144, 3, 512, 3, True),    # exact-size schedule, a second block with two live rows
+    (1, 2048, 1, 256, 1, False),     # one row
+    (300, 2176, 2, 1024, 2, False),  # 17 slabs: parts of unequal length
+])
+def test_few_jobs_deep_split_and_join_kernel(T, K, E, N, top_k, exact, device):
+    """Few up jobs for the chip and a long contraction: every up tile is split over up to 8 workgroups that
+    only store their partial sums, and a kernel of its own joins them and applies SwiGLU.  Against the
+    oracle, and bit for bit the same on a second call (the join adds the parts in part order)."""
+    import prime_moe
+    for split in (True, False):
+        _run_case(T, K, E, N, top_k, split, device, seed=T + K, use_op_align=not exact, exact=exact, hot_last=False)
+    g, x, w1, w2 = _inputs(T, K, E, N, device, T + K)
+    ids, wts = reference_routing(T, E, top_k, device, g, hot_last=False)
+    sched = torch.ops.prime_moe.moe_align(ids, E, 128, 1)
+    outs = []
+    for _ in range(2):
+        torch.empty((32 << 20,), dtype=torch.float32, device=device).fill_(float("nan"))  # dirty the allocator's blocks
+        out = torch.empty((T, K), dtype=torch.bfloat16, device=device)
+        prime_moe.fused_moe_bf16(x, w1, w2, *sched, wts, out, top_k, 128, 64, 4, 2, 1, 1, True)
+        outs.append(out)
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))

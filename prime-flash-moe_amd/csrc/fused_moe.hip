@@ -871,12 +871,14 @@ __device__ __forceinline__ void plan_tail_split(TailSplit &ts, int n_jobs, int n
     ts.per_xcd_tail = per_xcd_tail;
 }
 
+// Writes the work list entry of job `j` (of the (n_wt + per_job - 1) / per_job of the row tile; a workgroup
+// takes `per_job` consecutive weight tiles).
 __device__ __forceinline__ void emit_work(int4 *work, int n_wt, int per_job, int tile, int n_tiles, int first, int nb,
-                                          int e, const TailSplit *ts) {
+                                          int e, const TailSplit *ts, int j) {
     constexpr int GW = 8;
-    const int n_jobs = (n_wt + per_job - 1) / per_job;  // a workgroup takes `per_job` consecutive weight tiles
+    const int n_jobs = (n_wt + per_job - 1) / per_job;
     const int per_xcd = (n_tiles * n_jobs + 7) >> 3;
-    for (int j = 0; j < n_jobs; ++j) {
+    {
         const int wg = j / GW;
         const int gw = min(GW, n_jobs - wg * GW);
         const int l = wg * GW * n_tiles + tile * gw + (j - wg * GW);
@@ -975,12 +977,25 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
         ts_up.join_tab = join_tab;
         plan_tail_split(ts_up, up_counters != nullptr ? nt * ((n_wt_up + per_job_up - 1) / per_job_up) : 0, split_cus,
                         up_slabs, up_tail_jobs, kTailSlots, up_max_parts);
-        for (int t = tid; t < nt; t += 256) {
-            const int2 tl = tiles[t];
-            const int e = expert_ids[tl.x];
-            if (e < 0 || e >= num_experts) continue;  // nothing to compute for a block without an expert
-            emit_work(work_up, n_wt_up, per_job_up, t, nt, tl.x, tl.y, e, &ts_up);
-            emit_work(work_down, n_wt_down, per_job_down, t, nt, tl.x, tl.y, e, &ts);
+        const int jobs_up = (n_wt_up + per_job_up - 1) / per_job_up, jobs_down = (n_wt_down + per_job_down - 1) / per_job_down;
+        const int per_tile = jobs_up + jobs_down;
+        if (nt >= 64) {  // a row tile per thread and turn, its jobs one after the other
+            for (int t = tid; t < nt; t += 256) {
+                const int2 tl = tiles[t];
+                const int e = expert_ids[tl.x];
+                if (e < 0 || e >= num_experts) continue;  // nothing to compute for a block without an expert
+                for (int j = 0; j < jobs_up; ++j) emit_work(work_up, n_wt_up, per_job_up, t, nt, tl.x, tl.y, e, &ts_up, j);
+                for (int j = 0; j < jobs_down; ++j) emit_work(work_down, n_wt_down, per_job_down, t, nt, tl.x, tl.y, e, &ts, j);
+            }
+        } else {  // few row tiles for 256 threads: an entry per thread and turn (README shape: whole op 60 -> 56 us)
+            for (int i = tid; i < nt * per_tile; i += 256) {
+                const int t = i / per_tile, j = i - t * per_tile;
+                const int2 tl = tiles[t];
+                const int e = expert_ids[tl.x];
+                if (e < 0 || e >= num_experts) continue;
+                if (j < jobs_up) emit_work(work_up, n_wt_up, per_job_up, t, nt, tl.x, tl.y, e, &ts_up, j);
+                else emit_work(work_down, n_wt_down, per_job_down, t, nt, tl.x, tl.y, e, &ts, j - jobs_up);
+            }
         }
     }
     if (do_invert) {

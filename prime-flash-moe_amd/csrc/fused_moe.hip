@@ -66,6 +66,18 @@ struct MoeArgs {
 constexpr int kSkinnyRB = PMOE_SKINNY_RB;  // slab width of tiles with one live fragment
 constexpr int kPartRB = PMOE_PART_RB;      // of mxfp8 tiles with more, short of two full blocks
 
+// 16 bytes that this kernel writes or reads once (activation and y tiles, out): non-temporal, so that they
+// do not displace what the L2s could serve again (finalize: C3 -14 us, C4 -12 us; the two GEMM kernels gain
+// a few microseconds).
+__device__ __forceinline__ uint4 load_once(const void *p) {
+    const i32x4 v = __builtin_nontemporal_load(reinterpret_cast<const i32x4 *>(p));
+    return make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]);
+}
+__device__ __forceinline__ void store_once(void *p, uint4 q) {
+    i32x4 v;
+    v[0] = (int)q.x; v[1] = (int)q.y; v[2] = (int)q.z; v[3] = (int)q.w;
+    __builtin_nontemporal_store(v, reinterpret_cast<i32x4 *>(p));
+}
 constexpr int kActPitchBf16 = 272;  // 128 bf16 + 16 B pad: 16-byte aligned rows, 2-way conflicts at most
 constexpr int kActPitchFp8 = 144;   // 128 e4m3 + 16 B pad
 
@@ -79,6 +91,7 @@ constexpr int kActPitchFp8 = 144;   // 128 e4m3 + 16 B pad
 struct Job {
     int first, nb, wt, e, n_sub;
     int part, parts, slot;
+    bool w_once;  // no other row tile of this expert: nobody else reads the weight rows of this job
 };
 
 // Workgroup id -> job: one load from the work list, which the prologue lays out by workgroup id (see
@@ -94,6 +107,7 @@ __device__ __forceinline__ bool resolve_job(const MoeArgs &a, Job &j) {
     j.part = w.z & 0xf;
     j.parts = (w.z >> 4) & 0xf;
     j.slot = w.z >> 8;
+    j.w_once = (w.w & 1) != 0;
     return true;
 }
 
@@ -222,7 +236,7 @@ __device__ __forceinline__ void store_y_tile(const YDst &d, const char *tile, in
             const int dst_row = d.by_pair ? pair[row] : row;
             if (dst_row >= 0) {
                 const uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kYPitch + c * 16);
-                *reinterpret_cast<uint4 *>(d.base + dst_row * d.pitch + c * 16) = v;
+                store_once(d.base + dst_row * d.pitch + c * 16, v);
             }
         }
     }
@@ -288,7 +302,7 @@ __device__ __forceinline__ void store_act_tile(const MoeArgs &a, const char *til
             const int row = (gt >> 4) + 16 * i;
             if (row < 32 * ntf) {
                 uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchBf16 + c * 16);
-                *reinterpret_cast<uint4 *>(a.act + ((row0 + row) * H + h0) * 2 + c * 16) = v;
+                store_once(a.act + ((row0 + row) * H + h0) * 2 + c * 16, v);
             }
         }
     } else {
@@ -298,7 +312,7 @@ __device__ __forceinline__ void store_act_tile(const MoeArgs &a, const char *til
             const int row = (gt >> 3) + 32 * i;
             if (i < ntf) {
                 uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchFp8 + c * 16);
-                *reinterpret_cast<uint4 *>(a.act + (row0 + row) * H + h0 + c * 16) = v;
+                store_once(a.act + (row0 + row) * H + h0 + c * 16, v);
             }
         }
         if (gt < 32 * ntf)
@@ -375,7 +389,7 @@ __device__ __forceinline__ bool join_parts(const MoeArgs &a, const Job &j, f32x1
 template <int DT, int RB, bool FULL, typename TokOff, typename TokScOff, typename WScOff>
 __device__ __forceinline__ void setup_ring_loader(ring::Loader<RB> &ld, const ring::Layout &lay, int tid,
                                                   uint32_t w_pitch, int ntf0, int ntf1, const RowInfo<2> &ri,
-                                                  TokOff tok_row_off,
+                                                  bool w_once, TokOff tok_row_off,
                                                   const uint8_t *tok_sc_base, TokScOff tok_sc_off,
                                                   const uint8_t *w_sc_base, WScOff w_sc_off) {
     using L = ring::Loader<RB>;
@@ -428,6 +442,7 @@ __device__ __forceinline__ void setup_ring_loader(ring::Loader<RB> &ld, const ri
 #pragma unroll
     for (int q = 0; q < L::N; ++q) lps += (ld.tok_dst[0][q] >= 0) + (ld.tok_dst[1][q] >= 0);
     ld.lps = lps;
+    ld.w_once = w_once;
     ld.make_uniform();
 }
 
@@ -473,7 +488,7 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, const Job &job, R
     const uint32_t row_bytes = (uint32_t)(K * ES);
     const int kb = K >> 5, kt128 = K >> 7;
     setup_ring_loader<DT, RB, FULL>(
-        ld, lay, tid, row_bytes, ntf0, ntf1, ri,
+        ld, lay, tid, row_bytes, ntf0, ntf1, ri, job.w_once,
         [&](int row) { return (uint32_t)max(ri.tok[row], 0) * row_bytes; },
         reinterpret_cast<const uint8_t *>(a.xs_tiled + (int64_t)first * kt128 * kBlockRows),
         [&](int row) { return (uint32_t)(((row >> 7) * kt128 * kBlockRows + (row & 127)) * 4); },
@@ -652,7 +667,7 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, const Job &job,
     };
     set_weights(k0);
     setup_ring_loader<DT, RB, FULL>(
-        ld, lay, tid, row_bytes, ntf0, ntf1, ri, [&](int row) { return (uint32_t)row * row_bytes; },
+        ld, lay, tid, row_bytes, ntf0, ntf1, ri, job.w_once, [&](int row) { return (uint32_t)row * row_bytes; },
         reinterpret_cast<const uint8_t *>(a.act_scales + (int64_t)first * ht128 * kBlockRows),
         [&](int row) { return (uint32_t)(((row >> 7) * ht128 * kBlockRows + (row & 127)) * 4); },
         a.w2_scales + (int64_t)e * K * hb,
@@ -837,7 +852,8 @@ __global__ __launch_bounds__(256) void moe_up_join_kernel(MoeArgs a) {
 // is given to workgroup id 8 * (l mod per_xcd) + l / per_xcd: one XCD then runs a contiguous range of
 // the walk.  The entry carries everything the workgroup needs to start: x = first block | blocks << 28,
 // y = first weight tile | expert << 16 | (weight tiles - 1) << 26 (experts < 1024, up to 16 weight
-// tiles), z = part | parts << 4 | tail slot << 8 (see TailSplit).
+// tiles), z = part | parts << 4 | tail slot << 8 (see TailSplit), w = 1 if the row tile is the only one of
+// its expert.
 //
 // Workgroups start in the order of their ids, so the last `per_xcd_tail` positions of every XCD's range
 // are the jobs that would run while most CUs have nothing left to do.  The bf16 kernels split the
@@ -874,7 +890,7 @@ __device__ __forceinline__ void plan_tail_split(TailSplit &ts, int n_jobs, int n
 // Writes the work list entry of job `j` (of the (n_wt + per_job - 1) / per_job of the row tile; a workgroup
 // takes `per_job` consecutive weight tiles).
 __device__ __forceinline__ void emit_work(int4 *work, int n_wt, int per_job, int tile, int n_tiles, int first, int nb,
-                                          int e, const TailSplit *ts, int j) {
+                                          int e, const TailSplit *ts, int j, int flags) {
     constexpr int GW = 8;
     const int n_jobs = (n_wt + per_job - 1) / per_job;
     const int per_xcd = (n_tiles * n_jobs + 7) >> 3;
@@ -889,13 +905,13 @@ __device__ __forceinline__ void emit_work(int4 *work, int n_wt, int per_job, int
             const int slot = (pos - (per_xcd - ts->per_xcd_tail)) * 8 + xcd;  // number of the tail job
             const int z = (ts->parts << 4) | (slot << 8);
             const int extra = slot * (ts->parts - 1);
-            work[8 * pos + xcd] = make_int4(x, y, z, 0);
-            for (int p = 1; p < ts->parts; ++p) work[ts->extra_base + extra + p - 1] = make_int4(x, y, z | p, 0);
+            work[8 * pos + xcd] = make_int4(x, y, z, flags);
+            for (int p = 1; p < ts->parts; ++p) work[ts->extra_base + extra + p - 1] = make_int4(x, y, z | p, flags);
             if (ts->join_tab != nullptr) ts->join_tab[slot] = make_int4(x, wt, ts->parts, 0);
             if (ts->tail_tab != nullptr)
                 for (int b = 0; b < nb; ++b) ts->tail_tab[(first + b) * n_wt + wt] = (extra << 8) | (b << 4) | ts->parts;
         } else {
-            work[8 * pos + xcd] = make_int4(x, y, 1 << 4, 0);
+            work[8 * pos + xcd] = make_int4(x, y, 1 << 4, flags);
         }
     }
 }
@@ -979,13 +995,20 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
                         up_slabs, up_tail_jobs, kTailSlots, up_max_parts);
         const int jobs_up = (n_wt_up + per_job_up - 1) / per_job_up, jobs_down = (n_wt_down + per_job_down - 1) / per_job_down;
         const int per_tile = jobs_up + jobs_down;
+        // 1 if row tile t is the only one of its expert e (then nobody else reads that expert's weight rows)
+        auto only_tile = [&](int t, int e) {
+            const bool before = t > 0 && expert_ids[tiles[t - 1].x] == e;
+            const bool after = t + 1 < nt && expert_ids[tiles[t + 1].x] == e;
+            return (before || after) ? 0 : 1;
+        };
         if (nt >= 64) {  // a row tile per thread and turn, its jobs one after the other
             for (int t = tid; t < nt; t += 256) {
                 const int2 tl = tiles[t];
                 const int e = expert_ids[tl.x];
                 if (e < 0 || e >= num_experts) continue;  // nothing to compute for a block without an expert
-                for (int j = 0; j < jobs_up; ++j) emit_work(work_up, n_wt_up, per_job_up, t, nt, tl.x, tl.y, e, &ts_up, j);
-                for (int j = 0; j < jobs_down; ++j) emit_work(work_down, n_wt_down, per_job_down, t, nt, tl.x, tl.y, e, &ts, j);
+                const int fl = only_tile(t, e);
+                for (int j = 0; j < jobs_up; ++j) emit_work(work_up, n_wt_up, per_job_up, t, nt, tl.x, tl.y, e, &ts_up, j, fl);
+                for (int j = 0; j < jobs_down; ++j) emit_work(work_down, n_wt_down, per_job_down, t, nt, tl.x, tl.y, e, &ts, j, fl);
             }
         } else {  // few row tiles for 256 threads: an entry per thread and turn (README shape: whole op 60 -> 56 us)
             for (int i = tid; i < nt * per_tile; i += 256) {
@@ -993,8 +1016,9 @@ __global__ __launch_bounds__(256) void moe_prologue_kernel(const int32_t *expert
                 const int2 tl = tiles[t];
                 const int e = expert_ids[tl.x];
                 if (e < 0 || e >= num_experts) continue;
-                if (j < jobs_up) emit_work(work_up, n_wt_up, per_job_up, t, nt, tl.x, tl.y, e, &ts_up, j);
-                else emit_work(work_down, n_wt_down, per_job_down, t, nt, tl.x, tl.y, e, &ts, j - jobs_up);
+                const int fl = only_tile(t, e);
+                if (j < jobs_up) emit_work(work_up, n_wt_up, per_job_up, t, nt, tl.x, tl.y, e, &ts_up, j, fl);
+                else emit_work(work_down, n_wt_down, per_job_down, t, nt, tl.x, tl.y, e, &ts, j - jobs_up, fl);
             }
         }
     }
@@ -1099,7 +1123,7 @@ __global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int3
                 const int p = t * top_k + r0 + g;
                 if (row[g] >= 0) {
                     w[g] = topk_w[p];
-                    q[g] = *reinterpret_cast<const uint4 *>(y + ((int64_t)p * K + 8 * c) * 2);
+                    q[g] = load_once(y + ((int64_t)p * K + 8 * c) * 2);
                 }
             }
 #pragma unroll
@@ -1127,7 +1151,7 @@ __global__ __launch_bounds__(256) void finalize_kernel(const char *y, const int3
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) o[j] = pack2_bf16(v[2 * j], v[2 * j + 1]);
-        out[i] = make_uint4(o[0], o[1], o[2], o[3]);
+        store_once(out + i, make_uint4(o[0], o[1], o[2], o[3]));
     }
 }
 

@@ -64,7 +64,7 @@ struct MoeArgs {
 #define PMOE_PART_RB 128
 #endif
 constexpr int kSkinnyRB = PMOE_SKINNY_RB;  // slab width of tiles with one live fragment
-constexpr int kPartRB = PMOE_PART_RB;      // of mxfp8 tiles with more, short of two full blocks
+constexpr int kPartRB = PMOE_PART_RB;      // of mxfp8 tiles with more
 
 // 16 bytes that this kernel writes or reads once (activation and y tiles, out): non-temporal, so that they
 // do not displace what the L2s could serve again (finalize: C3 -14 us, C4 -12 us; the two GEMM kernels gain
@@ -386,7 +386,7 @@ __device__ __forceinline__ bool join_parts(const MoeArgs &a, const Job &j, f32x1
 // K tile lies 512 bytes on in both (blocked weight scales, tiled token-side scales).  Only the live 32-row
 // fragments of the two blocks (ntf0, ntf1 of them) are copied; they are packed one after the other in
 // the stage (see ring::Layout).
-template <int DT, int RB, bool FULL, typename TokOff, typename TokScOff, typename WScOff>
+template <int DT, int RB, typename TokOff, typename TokScOff, typename WScOff>
 __device__ __forceinline__ void setup_ring_loader(ring::Loader<RB> &ld, const ring::Layout &lay, int tid,
                                                   uint32_t w_pitch, int ntf0, int ntf1, const RowInfo<2> &ri,
                                                   bool w_once, TokOff tok_row_off,
@@ -405,9 +405,8 @@ __device__ __forceinline__ void setup_ring_loader(ring::Loader<RB> &ld, const ri
         const int frag = row0 >> 5;  // the instruction's rows lie in this 32-row fragment
         ld.tok_dst[0][q] = ld.tok_dst[1][q] = -1;
         ld.tok_off[0][q] = ld.tok_off[1][q] = 0;
-        // (the constant wait counts of full tiles assume every instruction: those copy all their rows)
-        ld.tok_live[0][q] = frag < ntf0 && (FULL || ri.tok[row] >= 0);
-        ld.tok_live[1][q] = frag < ntf1 && (FULL || ri.tok[kBlockRows + row] >= 0);
+        ld.tok_live[0][q] = frag < ntf0 && ri.tok[row] >= 0;
+        ld.tok_live[1][q] = frag < ntf1 && ri.tok[kBlockRows + row] >= 0;
         if (__ballot(ld.tok_live[0][q]) != 0) {
             ld.tok_dst[0][q] = row0 * RB;
             ld.tok_off[0][q] = tok_row_off(row) + gchunk;
@@ -461,7 +460,7 @@ __device__ __forceinline__ int slab_rotation(int n_slabs) {
 // columns [128 ht, 128 ht + 128).  LDS weight rows 0..127 are gate rows, 128..255 the matching up rows;
 // wave v of a group owns gate/up rows 32v..32v+31 so gate and up of one activation element sit in the
 // same lane and register.
-template <int DT, int RB, int NTF, bool FULL>
+template <int DT, int RB, int NTF>
 __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, const Job &job, RowInfo<2> &ri, char *lds,
                                              uint32_t *act_sc_lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
@@ -487,7 +486,7 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, const Job &job, R
     ld.w_base[1] = ld.w_base[0] + (int64_t)H * K * ES;
     const uint32_t row_bytes = (uint32_t)(K * ES);
     const int kb = K >> 5, kt128 = K >> 7;
-    setup_ring_loader<DT, RB, FULL>(
+    setup_ring_loader<DT, RB>(
         ld, lay, tid, row_bytes, ntf0, ntf1, ri, job.w_once,
         [&](int row) { return (uint32_t)max(ri.tok[row], 0) * row_bytes; },
         reinterpret_cast<const uint8_t *>(a.xs_tiled + (int64_t)first * kt128 * kBlockRows),
@@ -502,7 +501,7 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, const Job &job, R
     constexpr int kPitch = DT == DT_BF16 ? kActPitchBf16 : kActPitchFp8;
     char *tile = lds + grp * (kBlockRows * kPitch);
     uint32_t *sc_tile = act_sc_lds + grp * kBlockRows;
-    const int SB = ring::stage_bytes<DT, RB, FULL>(lay), NS = ring::stage_count<DT, RB, FULL>(lay);
+    const int SB = lay.stage_bytes, NS = lay.stages;
     // first stage clear of the activation tiles: the next weight tile's copies start there, under
     // the epilogue of this one
     const int epi_bytes = (ntf1 > 0 ? 2 : 1) * kBlockRows * kPitch;
@@ -512,9 +511,9 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, const Job &job, R
         f32x16 acc[2][4];
         zero_acc(acc);
         if (active)
-            ring::main_loop<DT, RB, NTF, true, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
+            ring::main_loop<DT, RB, NTF, true, true>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
         else
-            ring::main_loop<DT, RB, NTF, true, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
+            ring::main_loop<DT, RB, NTF, true, false>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
         if constexpr (DT == DT_BF16) {
             if (job.parts > 1 && !join_parts<NTF>(a, job, acc, active, reinterpret_cast<int *>(lds + 128 * 1024))) return;
         }
@@ -527,7 +526,7 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, const Job &job, R
             ld.make_uniform();
             stage0 = free0 < NS ? free0 : 0;
             n_pre = free0 < NS ? min(NS - 1, NS - free0) : 0;
-            ring::pre_issue<DT, RB, FULL>(ld, lay, lds, n_slabs, start, stage0, n_pre);
+            ring::pre_issue<DT, RB>(ld, lay, lds, n_slabs, start, stage0, n_pre);
         }
         if (active) swiglu_epilogue<DT, NTF>(acc, tile, sc_tile, w4, lane);
         __syncthreads();
@@ -610,7 +609,7 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {  // one weight tile per workgroup on this path (see launch_pipeline)
         j.n_sub = 1;
-        if (skinny) up_tile_ring<DT, kSkinnyRB, 1, false>(a, j, ri, lds, nullptr);
+        if (skinny) up_tile_ring<DT, kSkinnyRB, 1>(a, j, ri, lds, nullptr);
         else if (j.parts > 1) {  // one of the workgroups that share a tile of the kernel's tail
             if (ntf == 1) up_tile_wide_bf16<1, true>(a, j, ri, lds);
             else if (ntf == 2) up_tile_wide_bf16<2, true>(a, j, ri, lds);
@@ -620,18 +619,16 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
         else up_tile_wide_bf16<4, false>(a, j, ri, lds);
     } else {
         uint32_t *act_sc_lds = reinterpret_cast<uint32_t *>(lds + L::kActScaleOff);
-        const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-        if (ntf == 1) up_tile_ring<DT, kSkinnyRB, 1, false>(a, j, ri, lds, act_sc_lds);
-        else if (ntf == 2) up_tile_ring<DT, kPartRB, 2, false>(a, j, ri, lds, act_sc_lds);
-        else if (full) up_tile_ring<DT, 64, 4, true>(a, j, ri, lds, act_sc_lds);
-        else up_tile_ring<DT, kPartRB, 4, false>(a, j, ri, lds, act_sc_lds);
+        if (ntf == 1) up_tile_ring<DT, kSkinnyRB, 1>(a, j, ri, lds, act_sc_lds);
+        else if (ntf == 2) up_tile_ring<DT, kPartRB, 2>(a, j, ri, lds, act_sc_lds);
+        else up_tile_ring<DT, kPartRB, 4>(a, j, ri, lds, act_sc_lds);
     }
 }
 
 // Down kernel tile on the stage ring: y[rows, 256 cols of K] = act[rows, :H] . W2[e][cols, :H]^T, the
 // whole reduction over H inside the workgroup unless the job is one part of a split tail tile; the
 // routing weights are applied later, by finalize_kernel.
-template <int DT, int RB, int NTF, bool FULL>
+template <int DT, int RB, int NTF>
 __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, const Job &job, RowInfo<2> &ri, char *lds) {
     constexpr int ES = DT == DT_BF16 ? 2 : 1;
     const int first = job.first, kt = job.wt, n_sub = job.n_sub, e = job.e;
@@ -666,7 +663,7 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, const Job &job,
             ld.sc_off = (uint32_t)blocked_scale_off(min(k + 64 * (wave - 4) + lane, K - 1), 0, ht128);
     };
     set_weights(k0);
-    setup_ring_loader<DT, RB, FULL>(
+    setup_ring_loader<DT, RB>(
         ld, lay, tid, row_bytes, ntf0, ntf1, ri, job.w_once, [&](int row) { return (uint32_t)row * row_bytes; },
         reinterpret_cast<const uint8_t *>(a.act_scales + (int64_t)first * ht128 * kBlockRows),
         [&](int row) { return (uint32_t)(((row >> 7) * ht128 * kBlockRows + (row & 127)) * 4); },
@@ -676,7 +673,7 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, const Job &job,
     const int wrow[2] = {64 * w4, 64 * w4 + 32};
     const int start = slab_rotation<RB>(n_slabs);
     const int tok_region = grp ? lay.group1_off : 0;
-    const int SB = ring::stage_bytes<DT, RB, FULL>(lay), NS = ring::stage_count<DT, RB, FULL>(lay);
+    const int SB = lay.stage_bytes, NS = lay.stages;
     // the ring is free after main_loop (it ends with a barrier): its head holds the 128 x 256 output
     // tiles of the live groups (none for tiles of one fragment, which store from registers); the
     // next weight tile's copies start in the first stage clear of them, under this tile's epilogue
@@ -687,16 +684,16 @@ __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, const Job &job,
         f32x16 acc[2][4];
         zero_acc(acc);
         if (active)
-            ring::main_loop<DT, RB, NTF, true, true, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
+            ring::main_loop<DT, RB, NTF, true, true>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
         else
-            ring::main_loop<DT, RB, NTF, true, false, FULL>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
+            ring::main_loop<DT, RB, NTF, true, false>(acc, ld, lay, lds, n_slabs, wrow, lane, tok_region, start, stage0, n_pre);
         const bool more = sub + 1 < n_sub;
         if (more) {
             set_weights(k0 + kWRows);
             ld.make_uniform();
             stage0 = free0 < NS ? free0 : 0;
             n_pre = free0 < NS ? min(NS - 1, NS - free0) : 0;
-            ring::pre_issue<DT, RB, FULL>(ld, lay, lds, n_slabs, start, stage0, n_pre);
+            ring::pre_issue<DT, RB>(ld, lay, lds, n_slabs, start, stage0, n_pre);
         }
         const YDst dst = y_destination(a, job, grp, k0);
         if constexpr (NTF == 1) {
@@ -775,16 +772,14 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {  // one weight tile per workgroup on this path (see launch_pipeline)
         j.n_sub = 1;
-        if (skinny) down_tile_ring<DT, kSkinnyRB, 1, false>(a, j, ri, lds);
+        if (skinny) down_tile_ring<DT, kSkinnyRB, 1>(a, j, ri, lds);
         else if (ntf == 1) down_tile_wide_bf16<1>(a, j, ri, lds);
         else if (ntf == 2) down_tile_wide_bf16<2>(a, j, ri, lds);
         else down_tile_wide_bf16<4>(a, j, ri, lds);
     } else {
-        const bool full = ri.nvalid[0] > 96 && ri.nvalid[1] > 96;  // all four fragments of both blocks live
-        if (ntf == 1) down_tile_ring<DT, kSkinnyRB, 1, false>(a, j, ri, lds);
-        else if (ntf == 2) down_tile_ring<DT, kPartRB, 2, false>(a, j, ri, lds);
-        else if (full) down_tile_ring<DT, 64, 4, true>(a, j, ri, lds);
-        else down_tile_ring<DT, kPartRB, 4, false>(a, j, ri, lds);
+        if (ntf == 1) down_tile_ring<DT, kSkinnyRB, 1>(a, j, ri, lds);
+        else if (ntf == 2) down_tile_ring<DT, kPartRB, 2>(a, j, ri, lds);
+        else down_tile_ring<DT, kPartRB, 4>(a, j, ri, lds);
     }
 }
 

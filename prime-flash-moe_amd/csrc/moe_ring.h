@@ -65,15 +65,6 @@ __device__ __forceinline__ Layout make_layout(int ntf0, int ntf1, int budget) {
     l.stages = min(kMaxStages, budget / l.stage_bytes);
     return l;
 }
-// Compile-time geometry of the tile with two full blocks at RB = 64 (4 stages).
-template <int DT>
-struct FullCfg {
-    static constexpr int kStages = 4;
-    static constexpr int kTokRows = 256;
-    static constexpr int kWOff = kTokRows * 64;
-    static constexpr int kScaleOff = kWOff + kWRows * 64;
-    static constexpr int kStageBytes = kScaleOff + (DT == DT_FP8 ? (kTokRows + kWRows) * 4 : 0);
-};
 // LDS the ring may use, a multiple of 1 KB (the split kernels put their row table behind it).
 template <int DT>
 constexpr int ring_bytes() {
@@ -258,21 +249,12 @@ __device__ __forceinline__ void mma_fp8_step(f32x16 (&acc)[2][4], const char *to
         }
 }
 
-// Geometry of the ring in use: the constants of a full tile or the run-time layout.
-template <int DT, int RB, bool FULL>
-__device__ __forceinline__ int stage_bytes(const Layout &lay) {
-    return FULL ? FullCfg<DT>::kStageBytes : lay.stage_bytes;
-}
-template <int DT, int RB, bool FULL>
-__device__ __forceinline__ int stage_count(const Layout &lay) {
-    return FULL ? FullCfg<DT>::kStages : lay.stages;
-}
 // Issues slabs 0 .. n - 1 of a tile (at most stages - 1 of them, in rotated order from `start`) into
 // stages stage0, stage0 + 1, ...
-template <int DT, int RB, bool FULL>
+template <int DT, int RB>
 __device__ __forceinline__ void pre_issue(const Loader<RB> &ld, const Layout &lay, char *lds, int n_slabs, int start,
                                           int stage0, int n) {
-    const int SB = stage_bytes<DT, RB, FULL>(lay), NS = stage_count<DT, RB, FULL>(lay);
+    const int SB = lay.stage_bytes, NS = lay.stages;
     for (int s = 0; s < n; ++s) {
         if (s >= n_slabs) break;
         int slab = s + start;
@@ -290,25 +272,19 @@ __device__ __forceinline__ void pre_issue(const Loader<RB> &ld, const Layout &la
 // that run side by side and share rows then ask for different cache lines at any one time instead
 // of queueing on the same ones.  The sum over K does not depend on the order.
 //
-// FULL (RB = 64 only): the tile has two completely live blocks, so geometry and wait counts are
-// compile-time constants (`lay` must be that geometry); otherwise both are wave-uniform run-time
-// values and the wait count goes through a switch.
+// Geometry and wait counts are wave-uniform run-time values (the wait count goes through a switch).  A
+// variant for tiles of two full blocks with compile-time geometry, 64-byte slabs and 4 stages measured 2 - 3 %
+// slower on large mxfp8 batches than this loop with 128-byte slabs and 2 stages, and is gone.
 //
 // Slab 0 goes to stage `stage0`, the following ones to the stages behind it (wrapping).  `n_pre`: the
 // caller has already issued slabs 0 .. n_pre - 1 (see pre_issue; a workgroup that runs one tile
 // after another issues them under the previous tile's epilogue).
-template <int DT, int RB, int NTF, bool TRANSPOSED, bool COMPUTE, bool FULL>
+template <int DT, int RB, int NTF, bool TRANSPOSED, bool COMPUTE>
 __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader<RB> &ld, const Layout &lay, char *lds,
                                           int n_slabs, const int (&wrow)[2], int lane, int tok_region, int start,
                                           int stage0 = 0, int n_pre = 0) {
-    static_assert(!FULL || RB == 64, "the constant geometry is the 64-byte one");
-    using F = FullCfg<DT>;
-    const int SB = FULL ? F::kStageBytes : lay.stage_bytes;
-    const int NS = FULL ? F::kStages : lay.stages;
-    const int w_off = FULL ? F::kWOff : lay.w_off;
-    const int scale_off = FULL ? F::kScaleOff : lay.scale_off;
-    const int scale_tok_rows = FULL ? F::kTokRows : lay.scale_tok_rows;
-    constexpr int LPS_FULL = DT == DT_FP8 ? 5 : 4;
+    const int SB = lay.stage_bytes, NS = lay.stages;
+    const int w_off = lay.w_off, scale_off = lay.scale_off, scale_tok_rows = lay.scale_tok_rows;
     auto rot = [&](int s) {
         s += start;
         return s >= n_slabs ? s - n_slabs : s;
@@ -335,13 +311,7 @@ __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader<RB> 
     int fill_off = (stage0 == 0 ? NS - 1 : stage0 - 1) * SB;
     for (int kt = 0; kt < n_slabs; ++kt) {
         // slab kt has landed once at most the copies of the later slabs (up to NS - 2) are pending
-        if constexpr (FULL) {
-            if (kt + 2 < n_slabs) wait_and_barrier<2 * LPS_FULL>();
-            else if (kt + 1 < n_slabs) wait_and_barrier<LPS_FULL>();
-            else wait_and_barrier<0>();
-        } else {
-            wait_and_barrier_dyn(lps * min(NS - 2, n_slabs - 1 - kt));
-        }
+        wait_and_barrier_dyn(lps * min(NS - 2, n_slabs - 1 - kt));
         // the stage consumed in the previous iteration is free: everybody is past the barrier
         if (kt + NS - 1 < n_slabs) ld.issue(lds + fill_off, rot(kt + NS - 1));
         if constexpr (COMPUTE) {

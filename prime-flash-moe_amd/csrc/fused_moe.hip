@@ -551,6 +551,9 @@ struct SplitLds {
     static constexpr int kActScaleOff = kRowInfoOff + kRowInfoBytes;  // mxfp8 only
     static constexpr int kTotal = DT == DT_BF16 ? kRing : kActScaleOff + kBlockRows * 2 * 4;
     static_assert(sizeof(RowInfo<2>) <= kRowInfoBytes, "row table does not fit its slot");
+    // the epilogues reuse the head of the ring: two y tiles (down kernel) or two activation tiles (up kernel)
+    static_assert(2 * kBlockRows * kYPitch <= (DT == DT_BF16 ? kPairOff : kRing), "y tiles of the epilogue overrun their LDS");
+    static_assert(2 * kBlockRows * kActPitchBf16 <= kRing, "activation tiles of the epilogue overrun the ring");
     static_assert(DT != DT_BF16 || ring::ring_bytes<DT_BF16>() <= kRowInfoOff, "64-byte ring reaches the row table");
 };
 

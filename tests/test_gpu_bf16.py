@@ -163,6 +163,26 @@ def test_result_is_bitwise_reproducible(device):
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
 
 
+def test_experts_with_one_and_with_several_row_tiles(device):
+    # expert 0: 276 rows = a full row tile and a tail of 20 rows that reads the same weight rows; expert 1:
+    # 200 rows in one tile of two blocks; expert 2: 56 rows; expert 3: 20 rows, alone on its weight rows
+    # (decode-style tile, other cache policy of the weight copies); expert 4: none
+    import prime_moe
+    from test_gpu_mxfp8 import _routing_by_counts
+    counts, top_k = [276, 200, 56, 20, 0], 2
+    K, E, N = 1024, 5, 512
+    ids, wts = _routing_by_counts(counts, top_k, device, seed=6)
+    T = ids.shape[0]
+    g, x, w1, w2 = _inputs(T, K, E, N, device, seed=22)
+    sched = torch.ops.prime_moe.moe_align(ids, E, 128, 1)
+    for split in (True, False):
+        out = torch.zeros((T, K), dtype=torch.bfloat16, device=device)
+        prime_moe.fused_moe_bf16(x, w1, w2, *sched, wts, out, top_k, 128, 64, 4, 2, 1, 1, split)
+        torch.cuda.synchronize()
+        ref = O.fused_moe_dense(x.cpu(), w1.cpu(), w2.cpu(), ids.cpu(), wts.cpu())
+        assert rel_clamp(out.float().cpu(), ref, 1.0) <= BF16_GATE
+
+
 def test_block_without_expert_and_duplicate_pair(device):
     """Schedules the fused op must survive: a block whose expert id is out of range is not computed and
     its pairs contribute nothing (never whatever the workspace held); a pair id listed twice contributes

@@ -67,6 +67,44 @@ def _run_case(T, K, E, N, top_k, split, device, seed=0, use_op_align=True, exact
     return c, l2, rc1, rc10
 
 
+def _routing_by_counts(counts, top_k, device, seed):
+    """topk_ids with exactly counts[e] rows for expert e (sum = T * top_k, no expert twice in a token)."""
+    E, P = len(counts), sum(counts)
+    assert P % top_k == 0 and max(counts) <= P // top_k
+    T = P // top_k
+    # deal the experts' rows round the tokens, most frequent expert first: a token never gets one twice
+    order = sorted(range(E), key=lambda e: -counts[e])
+    flat = torch.tensor([e for e in order for _ in range(counts[e])], dtype=torch.int32)
+    ids = torch.empty((T, top_k), dtype=torch.int32)
+    for i in range(P):
+        ids[i % T, i // T] = flat[i]
+    g = torch.Generator().manual_seed(seed)
+    wts = torch.softmax(torch.randn((T, top_k), generator=g), dim=-1)
+    return ids.to(device), wts.to(device)
+
+
+@pytest.mark.parametrize("split", [True, False])
+def test_experts_with_one_and_with_several_row_tiles(split, device):
+    # expert 0: 700 rows = three row tiles that share its weight rows; experts 1 - 3: one row tile of two
+    # blocks each, whose weight rows only one workgroup per weight tile reads; expert 4: 20 rows; expert 5:
+    # none.  The weight copies of the two kinds differ in their cache policy.
+    import prime_moe
+    counts, top_k = [700, 250, 230, 200, 20, 0], 2
+    K, E, N = 1024, 6, 512
+    ids, wts = _routing_by_counts(counts, top_k, device, seed=5)
+    T = ids.shape[0]
+    g, a, deq = _quantised_inputs(T, K, E, N, device, seed=21)
+    sched = torch.ops.prime_moe.moe_align(ids, E, 128, 1)
+    out = torch.zeros((T, K), dtype=torch.bfloat16, device=device)
+    prime_moe.fused_moe_mxfp8(a["x"], a["x_scales"], a["w1"], a["w1_scales"], a["w2"], a["w2_scales"],
+                              *sched, wts, out, top_k, 128, 64, 4, 2, 1, split)
+    torch.cuda.synchronize()
+    ref = O.fused_moe_dense(deq["x"], deq["w1"], deq["w2"], ids.cpu(), wts.cpu(), act_mx=True)
+    got = out.float().cpu()
+    assert cosine(got, ref) >= MX_COS_GATE and rel_l2(got, ref) <= MX_RELL2_GATE
+    _elementwise_gates(got, ref)
+
+
 def _elementwise_gates(got, ref):
     """Element by element, in the reference's metric (test/test_mxfp8.py:168-191): a wrong scale byte or
     K block of a weight row fails these, whatever the norms say.

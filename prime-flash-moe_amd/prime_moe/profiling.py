@@ -2,13 +2,14 @@
 
     python prime-flash-moe_amd/prime_moe/profiling.py --config c2_mixtral_bf16 [--split 1] [--out profiles]
 
-Run from the repository root on a machine with the GPU.  Four profiler runs of ``bench.py`` on the same
+Run from the repository root on a machine with the GPU.  Five profiler runs of ``bench.py`` on the same
 workload, each a process of its own (the counter runs cannot share a process with a timed run):
 
   1. ``--kernel-trace --stats``                     average duration of every kernel
   2. ``--pmc FETCH_SIZE``  (+ ``--calibrate-copy``)  bytes fetched past the per-XCD L2s, per dispatch
   3. ``--pmc WRITE_SIZE``  (+ ``--calibrate-copy``)  bytes written past them
   4. ``--pmc`` eight SQ counters                    matrix-pipe busy cycles, LDS activity and conflicts, waits
+  5. ``--pmc`` four L2 (TCC) counters               reads past L2: requests, summed queue level, DRAM credit stalls
 
 ``--calibrate-copy`` adds launches of a plain 1 GiB copy kernel whose known traffic scales the two
 size counters.  The script writes ``<out>/split_pipeline_<config>.md`` (the commands, the raw per-kernel
@@ -33,6 +34,7 @@ KERNELS = ("moe_up_kernel", "moe_up_join_kernel", "moe_down_kernel", "finalize_k
            "copy_calibration_kernel")
 SQ_COUNTERS = ["SQ_BUSY_CYCLES", "SQ_VALU_MFMA_BUSY_CYCLES", "SQ_INSTS_VALU_MFMA_MOPS_{DT}", "SQ_LDS_BANK_CONFLICT",
                "SQ_ACTIVE_INST_LDS", "SQ_WAIT_INST_LDS", "SQ_WAVE_CYCLES", "SQ_WAIT_ANY"]
+EA_COUNTERS = ["TCC_EA0_RDREQ_sum", "TCC_EA0_RDREQ_LEVEL_sum", "TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum", "TCC_BUSY_sum"]
 GIB_KIB = 1048576.0
 
 
@@ -116,7 +118,9 @@ def main():
     d_write, _, _ = run_pass("write", ["--pmc", "WRITE_SIZE"], ["--steps", "3", "--warmup", "1", "--calibrate-copy", *common],
                           a.workdir, cmds)
     d_sq, _, _ = run_pass("sq", ["--pmc", *sq], ["--steps", "3", "--warmup", "1", *common], a.workdir, cmds)
+    d_ea, _, _ = run_pass("ea", ["--pmc", *EA_COUNTERS], ["--steps", "3", "--warmup", "1", *common], a.workdir, cmds)
     stats, fetch, write, sqc = kernel_stats(d_stats), counters(d_fetch), counters(d_write), counters(d_sq)
+    eac = counters(d_ea)
     cal_f = fetch.get("copy_calibration_kernel", {}).get("FETCH_SIZE", (GIB_KIB, 0))[0]
     cal_w = write.get("copy_calibration_kernel", {}).get("WRITE_SIZE", (GIB_KIB, 0))[0]
     f_scale, w_scale = GIB_KIB / cal_f, GIB_KIB / cal_w
@@ -131,8 +135,8 @@ def main():
               f"FETCH_SIZE reads {cal_f:,.0f} KiB for it (scale factor {f_scale:.2f}), WRITE_SIZE {cal_w:,.0f} KiB (scale factor {w_scale:.2f}).",
               "", "bench.py's own line of the traced run (profiler attached):", "", "    " + bench_line, "",
               "## Per kernel (means per dispatch)", "",
-              "| kernel | avg duration | fetched past L2 | written past L2 | sum | algorithmic bytes | rate | MFMA busy | LDS conflict cycles / LDS active | waiting on LDS |",
-              "|---|---|---|---|---|---|---|---|---|---|"]
+              "| kernel | avg duration | fetched past L2 | written past L2 | sum | algorithmic bytes | rate | MFMA busy | LDS conflict cycles / LDS active | waiting on LDS | read latency past L2 | DRAM credit stalls |",
+              "|---|---|---|---|---|---|---|---|---|---|---|---|"]
     figs = []
     for k in KERNELS[:5]:
         if k not in stats:
@@ -150,12 +154,19 @@ def main():
         wait_lds = c.get("SQ_WAIT_INST_LDS", 0.0) / c["SQ_WAVE_CYCLES"] if c.get("SQ_WAVE_CYCLES") else 0.0
         mfma_frac = mfma / busy if busy else 0.0
         ab = algorithmic.get(k)
+        e = {n.replace("_sum", ""): v[0] for n, v in eac.get(k, {}).items()}
+        ea_lat = e.get("TCC_EA0_RDREQ_LEVEL", 0.0) / e["TCC_EA0_RDREQ"] if e.get("TCC_EA0_RDREQ") else 0.0
+        ea_stall = e.get("TCC_EA0_RDREQ_DRAM_CREDIT_STALL", 0.0) / e["TCC_BUSY"] if e.get("TCC_BUSY") else 0.0
         lines.append(f"| {k} | {us:.1f} us | {fb / 1e9:.3f} GB | {wb / 1e9:.3f} GB | {(fb + wb) / 1e9:.3f} GB | "
-                     f"{(f'{ab / 1e9:.3f} GB' if ab else '')} | {(fb + wb) / us / 1e6:.2f} TB/s | {mfma_frac:.3f} | {conflict:.3f} | {wait_lds:.3f} |")
+                     f"{(f'{ab / 1e9:.3f} GB' if ab else '')} | {(fb + wb) / us / 1e6:.2f} TB/s | {mfma_frac:.3f} | {conflict:.3f} | {wait_lds:.3f} | "
+                     f"{ea_lat:.0f} L2 clk | {ea_stall:.4f} |")
         figs.append(f"{a.config} {k} avg_us {us:.1f} fetch_bytes {fb:.0f} write_bytes {wb:.0f} mfma_busy {mfma_frac:.4f} "
                     f"lds_conflict {conflict:.4f}")
     lines += ["", "MFMA busy = SQ_VALU_MFMA_BUSY_CYCLES (summed over SIMDs) / (SQ_BUSY_CYCLES (summed over shader engines) x SIMDs per",
               f"shader engine = {simds_per_se:.0f}): the share of the cycles a SIMD is busy in which its matrix pipe is.",
+              "Read latency past L2 = TCC_EA0_RDREQ_LEVEL / TCC_EA0_RDREQ (mean time a read that missed L2 is outstanding, in L2",
+              "clocks); DRAM credit stalls = TCC_EA0_RDREQ_DRAM_CREDIT_STALL / TCC_BUSY (share of the L2-busy cycles in which a",
+              "read could not be sent on for lack of DRAM credits: the memory side saturated).",
               "FETCH_SIZE counts what misses the per-XCD L2s, whether the memory-side cache or HBM serves it.  Algorithmic bytes:",
               "weights (+ scales) of the touched experts once, the routed rows of the token-side operand once, the output once.", "",
               "## Raw figures", ""]
@@ -163,7 +174,7 @@ def main():
         if k in stats:
             s = stats[k]
             lines.append(f"    {k}: calls {s['calls']} avg_ns {s['avg_ns']:.0f} min_ns {s['min_ns']:.0f} max_ns {s['max_ns']:.0f}")
-        for src in (fetch, write, sqc):
+        for src in (fetch, write, sqc, eac):
             for cname, (v, n) in sorted(src.get(k, {}).items()):
                 lines.append(f"    {k}: {cname} {v:.1f} (mean of {n} dispatches)")
     os.makedirs(a.out, exist_ok=True)

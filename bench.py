@@ -15,7 +15,9 @@ configuration and both values of `split` where the specification names both, tak
 headline run (`--headline-only` skips them), plus the router front-end next to the unfused sequence.
 
 `--sweep` runs the reference benchmark's token sweep against torch's grouped GEMM on this GPU and
-writes a CSV with the reference's columns (prime_moe/sweep.py).
+writes a CSV with the reference's columns (prime_moe/sweep.py); it takes the reference benchmark's
+knobs (--sweep-tokens, --sweep-dtypes, --experts, --top-k, --hidden, --inter, --balancedness, --seed,
+--graphs, --skip-naive).
 """
 from __future__ import annotations
 
@@ -297,6 +299,17 @@ def main():
     ap.add_argument("--sweep", action="store_true", help="token sweep against torch's grouped GEMM, CSV output")
     ap.add_argument("--sweep-out", default=os.path.join(ROOT, "gpurun_out", "sweep.csv"))
     ap.add_argument("--sweep-tokens", type=int, nargs="+", default=[4096, 8192, 16384, 32768, 65536, 131072])
+    # the reference benchmark's knobs (benchmark/benchmark.py:695-721), for --sweep only
+    ap.add_argument("--sweep-dtypes", nargs="+", choices=["bf16", "mxfp8"], default=["bf16", "mxfp8"])
+    ap.add_argument("--experts", type=int, default=32)
+    ap.add_argument("--top-k", type=int, default=4)
+    ap.add_argument("--hidden", type=int, default=2048, help="K, the model dim")
+    ap.add_argument("--inter", type=int, default=1024, help="per expert intermediate dim H; w1 has N = 2H rows")
+    ap.add_argument("--balancedness", type=float, default=1.0, help="1.0 = uniform routing, 0.0 = everything to expert 0")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--graphs", action=argparse.BooleanOptionalAction, default=False,
+                    help="time graph replays instead of eager calls (the reference's --cuda-graphs)")
+    ap.add_argument("--skip-naive", action="store_true", help="skip the per-expert loop baseline")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path is single-device, "
@@ -311,7 +324,10 @@ def main():
     if args.sweep:
         from prime_moe.sweep import run_sweep
         os.makedirs(os.path.dirname(os.path.abspath(args.sweep_out)), exist_ok=True)
-        rows = run_sweep(args.sweep_out, tokens=tuple(args.sweep_tokens), warmup=min(args.warmup, 10), iters=args.steps, log=log)
+        rows = run_sweep(args.sweep_out, tokens=tuple(args.sweep_tokens), dtypes=tuple(args.sweep_dtypes), E=args.experts,
+                         top_k=args.top_k, K=args.hidden, H=args.inter, warmup=min(args.warmup, 10), iters=args.steps,
+                         log=log, seed=args.seed, balancedness=args.balancedness, graphs=args.graphs,
+                         skip_naive=args.skip_naive)
         print(json.dumps({"sweep_csv": args.sweep_out, "rows": len(rows),
                           "speedup_min": min(r["speedup"] for r in rows), "speedup_max": max(r["speedup"] for r in rows)}))
         return

@@ -12,7 +12,11 @@ mxfp8 rows therefore use the same bf16 grouped baseline on the dequantised opera
 ``baseline_kind`` says which), and ``noreq_ms`` stays empty.
 
 Default grid = the reference's (benchmark.py:695-718): E=32, top_k=4, K=2048, H=1024,
-tokens 4096 ... 131072, both dtypes, split=True, median of per-iteration event timings.
+tokens 4096 ... 131072, both dtypes, split=True, median of per-iteration event timings.  Like the
+reference's, the run can be shaped from the command line (``bench.py --sweep``): experts, top_k, hidden and
+intermediate size, ``balancedness`` of the routing (benchmark.py:116-121: every (token, slot) draws its
+expert from ``b * uniform + (1 - b) * all-to-expert-0``, with replacement), seed, and whether the timed
+callables are graph replays (benchmark.py:355-370, the reference's default) or eager calls.
 """
 from __future__ import annotations
 
@@ -46,6 +50,37 @@ def median_ms(fn, warmup: int, iters: int) -> float:
     return statistics.median(times)
 
 
+def graphed(fn, warmup: int = 3):
+    """`fn` captured into a graph after a warm-up on a side stream; None if the capture fails (the
+    reference's recipe, benchmark.py:355-370: the caller then times `fn` eagerly)."""
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(warmup):
+                fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        return g.replay
+    except Exception:
+        torch.cuda.synchronize()
+        return None
+
+
+def generate_topk_ids(E: int, tokens: int, top_k: int, balancedness: float, gen: torch.Generator) -> torch.Tensor:
+    """The reference benchmark's routing (benchmark.py:116-121): 1.0 = uniform, 0.0 = everything to expert 0;
+    slots are drawn independently, so a token may name an expert twice."""
+    dev = gen.device
+    uniform = torch.ones(E, device=dev) / E
+    skewed = torch.zeros(E, device=dev)
+    skewed[0] = 1.0
+    probs = balancedness * uniform + (1.0 - balancedness) * skewed
+    return torch.multinomial(probs, tokens * top_k, replacement=True, generator=gen).view(tokens, top_k).to(torch.int32)
+
+
 def grouped_inputs(x, topk_ids, topk_weights, E):
     """Rows in expert order (stable), their tokens, routing weights and the group ends."""
     top_k = topk_ids.shape[1]
@@ -76,14 +111,15 @@ def naive_forward(xg, w1, w2, counts, wg):
 
 
 def run_one(dtype: str, tokens: int, E: int, K: int, H: int, top_k: int, split: bool, warmup: int, iters: int,
-            check: bool, seed: int = 0, skip_naive: bool = False) -> dict:
+            check: bool, seed: int = 0, skip_naive: bool = False, balancedness: float = 1.0, graphs: bool = False,
+            log=None) -> dict:
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev).manual_seed(seed)
     N = 2 * H
     x = (torch.randn((tokens, K), device=dev, generator=g) * 0.05).to(torch.bfloat16)
     w1 = (torch.randn((E, N, K), device=dev, generator=g) * 0.05).to(torch.bfloat16)
     w2 = (torch.randn((E, K, H), device=dev, generator=g) * 0.05).to(torch.bfloat16)
-    topk_ids = torch.randint(0, E, (tokens, top_k), device=dev, generator=g, dtype=torch.int32)
+    topk_ids = generate_topk_ids(E, tokens, top_k, balancedness, g)
     topk_weights = torch.softmax(torch.randn((tokens, top_k), device=dev, generator=g), -1)
     sched = torch.ops.prime_moe.moe_align(topk_ids, E, 128, 1)
     out = torch.zeros((tokens, K), dtype=torch.bfloat16, device=dev)
@@ -131,9 +167,16 @@ def run_one(dtype: str, tokens: int, E: int, K: int, H: int, top_k: int, split: 
         torch.cuda.synchronize()
         diff = (ref.float() - got).abs()
         max_abs, rel = float(diff.max()), float((diff / ref.float().abs().clamp_min(1.0)).max())
-    baseline_ms = median_ms(baseline, warmup, iters)
-    naive_ms = float("nan") if skip_naive else median_ms(naive, warmup, iters)
-    fused_ms = median_ms(step, warmup, iters)
+    timed = {"baseline": baseline, "naive": naive, "fused": step}
+    if graphs:
+        for name in ("baseline", "fused") + (() if skip_naive else ("naive",)):
+            replay = graphed(timed[name])
+            if replay is None and log is not None:
+                log(f"  note: graph capture failed for the {name} callable, timing it eagerly")
+            timed[name] = replay or timed[name]
+    baseline_ms = median_ms(timed["baseline"], warmup, iters)
+    naive_ms = float("nan") if skip_naive else median_ms(timed["naive"], warmup, iters)
+    fused_ms = median_ms(timed["fused"], warmup, iters)
     flops = 3.0 * tokens * top_k * K * N  # reference's model, benchmark.py:389-391
     tf = lambda ms: flops / (ms * 1e-3) / 1e12
     return {"dtype": dtype, "tokens": tokens, "E": E, "K": K, "N": N, "top_k": top_k, "naive_ms": naive_ms,
@@ -144,15 +187,18 @@ def run_one(dtype: str, tokens: int, E: int, K: int, H: int, top_k: int, split: 
 
 
 def run_sweep(path: str, tokens=(4096, 8192, 16384, 32768, 65536, 131072), dtypes=("bf16", "mxfp8"), E=32, top_k=4,
-              K=2048, H=1024, split=True, warmup=10, iters=50, check=True, log=print):
+              K=2048, H=1024, split=True, warmup=10, iters=50, check=True, log=print, seed=0, balancedness=1.0,
+              graphs=False, skip_naive=False):
     rows = []
     for dtype in dtypes:
         for t in tokens:
-            r = run_one(dtype, t, E, K, H, top_k, split, warmup, iters, check)
+            r = run_one(dtype, t, E, K, H, top_k, split, warmup, iters, check, seed=seed, skip_naive=skip_naive,
+                        balancedness=balancedness, graphs=graphs, log=log)
             rows.append(r)
             log(f"{dtype:6s} tokens {t:7d}: fused {r['fused_ms']:8.3f} ms ({r['fused_tflops']:7.1f} TFLOP/s)  "
                 f"{r['baseline_kind']} {r['baseline_ms']:8.3f} ms  speedup {r['speedup']:.2f}x  "
-                f"naive loop {r['naive_ms']:8.3f} ms  max_abs {r['max_abs']:.3g} rel {r['rel']:.3g}")
+                f"naive loop {r['naive_ms']:8.3f} ms  max_abs {r['max_abs']:.3g} rel {r['rel']:.3g}"
+                + ("  (graph replays)" if graphs else ""))
             torch.cuda.empty_cache()
     with open(path, "w", newline="") as f:
         w = csv.DictWriter(f, fieldnames=COLUMNS)

@@ -57,14 +57,17 @@ struct MoeArgs {
     int n_wtiles;  // weight tiles along the free dimension: H/128 (up) or ceil(K/256) (down)
 };
 
+// Slab width (bytes per row and slab) of the stage-ring tiles.  128: every request is a whole cache line.
+// 64 (twice the stages in the same LDS) stays selectable at build time for measurements: with the
+// non-temporal weight copies it runs the decode shape 32 % and the DeepSeek-like prefill 40 % slower.
 #ifndef PMOE_SKINNY_RB
 #define PMOE_SKINNY_RB 128
 #endif
 #ifndef PMOE_PART_RB
 #define PMOE_PART_RB 128
 #endif
-constexpr int kSkinnyRB = PMOE_SKINNY_RB;  // slab width of tiles with one live fragment
-constexpr int kPartRB = PMOE_PART_RB;      // of mxfp8 tiles with more
+constexpr int kSkinnyRB = PMOE_SKINNY_RB;  // tiles with one live fragment
+constexpr int kPartRB = PMOE_PART_RB;      // mxfp8 tiles with more
 
 // 16 bytes that this kernel writes or reads once (activation and y tiles, out): non-temporal, so that they
 // do not displace what the L2s could serve again (finalize: C3 -14 us, C4 -12 us; the two GEMM kernels gain

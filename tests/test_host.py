@@ -230,3 +230,18 @@ def test_workload_table_matches_benchmark_configs():
     assert round(CONFIGS["c5_decode_mxfp8"].flops / 1e9, 1) == 45.1
     c4 = CONFIGS["c4_dsv3_mxfp8"]
     assert c4.weight_bytes_per_expert() == (4096 * 7168 + 7168 * 2048) * 33 // 32
+
+
+def test_sweep_routing_and_columns_on_the_host():
+    # the benchmark harness's routing generator (reference: benchmark/benchmark.py:116-121) and its CSV
+    # header (benchmark.py:523-543) need no GPU
+    from prime_moe import sweep
+    g = torch.Generator().manual_seed(0)
+    assert int(sweep.generate_topk_ids(16, 2048, 4, 0.0, g).max()) == 0
+    ids = sweep.generate_topk_ids(16, 2048, 4, 0.5, g)
+    assert ids.dtype == torch.int32 and ids.shape == (2048, 4) and 0 <= int(ids.min()) and int(ids.max()) < 16
+    assert 0.47 < float((ids == 0).float().mean()) < 0.60  # 0.5 + 0.5 / 16
+    assert sweep.COLUMNS[:6] == ["dtype", "tokens", "E", "K", "N", "top_k"]
+    assert sweep.COLUMNS[6:19] == ["naive_ms", "baseline_ms", "noreq_ms", "fused_ms", "speedup", "speedup_noreq",
+                                   "speedup_naive", "naive_tflops", "baseline_tflops", "fused_tflops", "max_abs", "rel",
+                                   "naive_max_abs"]

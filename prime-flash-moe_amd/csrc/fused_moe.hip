@@ -790,12 +790,14 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
 }
 
 // Joins the parts of split up tiles when the up kernel left them in memory (a.deep_join).  One workgroup of
-// 4 waves per (job, row block of the tile, 32-row fragment): thread (w4, lane) takes over what thread
-// (block, w4, lane) of an up workgroup holds for that fragment, 16 gate and 16 up sums, adds the parts in
-// part order, applies SwiGLU and writes its 4 x 4 activation values.  Same sums in the same order as
-// join_parts, so the same bits.
+// 4 waves per (job, row block of the tile, 32-row fragment, quarter of the accumulator registers): thread
+// (w4, lane) takes over registers 4q .. 4q + 3 of what thread (block, w4, lane) of an up workgroup holds for
+// that fragment, gate and up sums, adds the parts in part order, applies SwiGLU and writes its 4 activation
+// values.  Same sums in the same order as join_parts, so the same bits.  All loads of a thread (the row's
+// sorted id, which only decides whether anything is written, and the 2 x parts partial sums) are in flight
+// together: the kernel is one memory latency long.
 __global__ __launch_bounds__(256) void moe_up_join_kernel(MoeArgs a) {
-    const int slot = blockIdx.x >> 3, grp = (blockIdx.x >> 2) & 1, t = blockIdx.x & 3;
+    const int slot = blockIdx.x >> 5, grp = (blockIdx.x >> 4) & 1, t = (blockIdx.x >> 2) & 3, q = blockIdx.x & 3;
     const int4 jt = a.join_tab[slot];
     const int parts = jt.z;
     if (parts < 2) return;
@@ -803,44 +805,33 @@ __global__ __launch_bounds__(256) void moe_up_join_kernel(MoeArgs a) {
     if (grp >= nb) return;
     const int tid = threadIdx.x, lane = tid & 63, w4 = tid >> 6;
     const int r = lane & 31, half = lane >> 5;
-    // a fragment without a live row has nothing to write (every wave looks at the same 32 rows)
     const int64_t srow0 = (int64_t)(first + grp) * kBlockRows + 32 * t;
-    {
-        const int64_t s = srow0 + r;
-        const int p = s < a.sorted_num ? a.sorted_ids[s] : -1;
-        if (__ballot(p >= 0 && p / a.top_k < a.M) == 0) return;
-    }
+    const int64_t s = srow0 + r;
+    const int p_row = s < a.sorted_num ? a.sorted_ids[s] : -1;
     const int src_tid = grp * 256 + tid;
-    float g[16], u[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) g[i] = u[i] = 0.f;
     const float4 *base = reinterpret_cast<const float4 *>(a.up_partials);
+    float4 vg[kDeepParts], vu[kDeepParts];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        float4 vg[kDeepParts], vu[kDeepParts];
+    for (int p = 0; p < kDeepParts; ++p)
+        if (p < parts) {
+            const float4 *src = base + ((int64_t)(slot * a.up_part_stride + p) * 32) * 512;
+            vg[p] = src[((0 * 4 + t) * 4 + q) * 512 + src_tid];
+            vu[p] = src[((1 * 4 + t) * 4 + q) * 512 + src_tid];
+        }
+    // a fragment without a live row has nothing to write (every wave looks at the same 32 rows)
+    if (__ballot(p_row >= 0 && p_row / a.top_k < a.M) == 0) return;
+    float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int p = 0; p < kDeepParts; ++p)
-            if (p < parts) {
-                const float4 *src = base + ((int64_t)(slot * a.up_part_stride + p) * 32) * 512;
-                vg[p] = src[((0 * 4 + t) * 4 + q) * 512 + src_tid];
-                vu[p] = src[((1 * 4 + t) * 4 + q) * 512 + src_tid];
-            }
-#pragma unroll
-        for (int p = 0; p < kDeepParts; ++p)
-            if (p < parts) {
-                g[4 * q] += vg[p].x; g[4 * q + 1] += vg[p].y; g[4 * q + 2] += vg[p].z; g[4 * q + 3] += vg[p].w;
-                u[4 * q] += vu[p].x; u[4 * q + 1] += vu[p].y; u[4 * q + 2] += vu[p].z; u[4 * q + 3] += vu[p].w;
-            }
-    }
-    char *dst = a.act + ((srow0 + r) * a.H + ht * 128) * 2;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const int hl = 32 * w4 + 8 * q + 4 * half;  // tile-local activation column, as in swiglu_epilogue
-        uint2 pk;
-        pk.x = pack2_bf16(swiglu(g[4 * q], u[4 * q]), swiglu(g[4 * q + 1], u[4 * q + 1]));
-        pk.y = pack2_bf16(swiglu(g[4 * q + 2], u[4 * q + 2]), swiglu(g[4 * q + 3], u[4 * q + 3]));
-        *reinterpret_cast<uint2 *>(dst + hl * 2) = pk;
-    }
+    for (int p = 0; p < kDeepParts; ++p)
+        if (p < parts) {
+            g[0] += vg[p].x; g[1] += vg[p].y; g[2] += vg[p].z; g[3] += vg[p].w;
+            u[0] += vu[p].x; u[1] += vu[p].y; u[2] += vu[p].z; u[3] += vu[p].w;
+        }
+    const int hl = 32 * w4 + 8 * q + 4 * half;  // tile-local activation column, as in swiglu_epilogue
+    uint2 pk;
+    pk.x = pack2_bf16(swiglu(g[0], u[0]), swiglu(g[1], u[1]));
+    pk.y = pack2_bf16(swiglu(g[2], u[2]), swiglu(g[3], u[3]));
+    *reinterpret_cast<uint2 *>(a.act + ((srow0 + r) * a.H + ht * 128 + hl) * 2) = pk;
 }
 
 // Walk order of the tiles of one kernel: [group of 8 weight tiles][row tile][weight tile in group].
@@ -1290,7 +1281,7 @@ static int launch_pipeline(MoeArgs a, const SchedBuffers &sb, void *out, int spl
         a.work = sb.work_up;
         if (mask & PMOE_PHASE_UP) {
             hipLaunchKernelGGL((moe_up_kernel<DT>), dim3(grid_up), dim3(512), 0, s, a);
-            if (a.deep_join) hipLaunchKernelGGL(moe_up_join_kernel, dim3(sb.up_tail_jobs * 8), dim3(256), 0, s, a);
+            if (a.deep_join) hipLaunchKernelGGL(moe_up_join_kernel, dim3(sb.up_tail_jobs * 32), dim3(256), 0, s, a);
         }
         MoeArgs d = a;
         d.n_wtiles = n_wt_down;

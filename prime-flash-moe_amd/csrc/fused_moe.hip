@@ -615,7 +615,12 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {  // one weight tile per workgroup on this path (see launch_pipeline)
         j.n_sub = 1;
-        if (skinny) up_tile_ring<DT, kSkinnyRB, 1>(a, j, ri, lds, nullptr);
+        if (skinny) {
+            // (an expert's last few rows: whatever its other row tiles fetched of these weight rows has left the
+            // caches by the time this tile runs, so its copies are non-temporal too; C2 -0.6 %, no loss elsewhere)
+            j.w_once = true;
+            up_tile_ring<DT, kSkinnyRB, 1>(a, j, ri, lds, nullptr);
+        }
         else if (j.parts > 1) {  // one of the workgroups that share a tile of the kernel's tail
             if (ntf == 1) up_tile_wide_bf16<1, true>(a, j, ri, lds);
             else if (ntf == 2) up_tile_wide_bf16<2, true>(a, j, ri, lds);
@@ -778,7 +783,10 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeArgs a) {
     const bool skinny = ntf == 1 && ri.nvalid[1] == 0;
     if constexpr (DT == DT_BF16) {  // one weight tile per workgroup on this path (see launch_pipeline)
         j.n_sub = 1;
-        if (skinny) down_tile_ring<DT, kSkinnyRB, 1>(a, j, ri, lds);
+        if (skinny) {
+            j.w_once = true;  // (see moe_up_kernel)
+            down_tile_ring<DT, kSkinnyRB, 1>(a, j, ri, lds);
+        }
         else if (ntf == 1) down_tile_wide_bf16<1>(a, j, ri, lds);
         else if (ntf == 2) down_tile_wide_bf16<2>(a, j, ri, lds);
         else down_tile_wide_bf16<4>(a, j, ri, lds);

@@ -17,7 +17,7 @@ CSRC = os.path.join(os.path.dirname(HERE), "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_NAME = "libprime_moe_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["api.hip", "moe_align.hip", "route.hip", "quantize_mx.hip", "fused_moe.hip"]
+SOURCES = ["api.hip", "moe_align.hip", "route.hip", "quantize_mx.hip", "fused_moe.hip", "fused_moe_bf16.hip"]
 ARCH = "gfx950"
 
 # Packed-fp32 VALU forms are switched off for every device compile.
@@ -52,7 +52,7 @@ def _compile(src: str, verbose: bool) -> str:
 
 def build(verbose: bool = True) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=4) as pool:
+    with ThreadPoolExecutor(max_workers=6) as pool:
         objs = list(pool.map(lambda s: _compile(s, verbose), SOURCES))
     cmd = [hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", LIB_PATH]
     if verbose:

@@ -33,23 +33,21 @@ def test_library_exports_every_declared_symbol():
 def test_workspace_query_and_c_side_validation_need_no_gpu():
     from prime_moe import _native
     lib = _native.load()
-    # header (256 B) + counters of split up jobs (256 B) + their join table (1 KB) + row-tile list (8 B per
-    # block) + the two work lists (16 B per block and weight tile, plus 192 entries each for the parts of
-    # split tail jobs) + [bf16: table of the split down tiles (4 B per block and down weight tile) + partial
-    # tiles of 256 x 256 bf16 for the split down jobs (3 per job, at most 192) + fp32 partial accumulators of
-    # the split up jobs (no more than there are jobs, at most 64) x 4 parts, or x 8 parts when at most 32
-    # jobs are joined by a kernel of their own] + inverse of the sorted order (4 B per pair) + y (one row of
-    # K bf16 per pair) + act (rows*H) [+ mxfp8: act scales + re-tiled x scales], each rounded to 256 B; the
-    # same for both values of split
+    # bf16: plan (256 B) + run list and the two tables of row tiles (16 B per block + 1 each) + fp32 partial sums of
+    # the deep contraction split when the problem has at most 32 (block, up weight tile) pairs and K >= 2048
+    # (8 parts x 32 KB per fragment and weight tile) + inverse of the sorted order (4 B per pair) + y (one row of
+    # K bf16 per pair) + act (rows * H bf16), each rounded to 256 B; the same for both values of split
     assert lib.pmoe_fused_moe_bf16_workspace_bytes(256, 4096, 512, 8, 2048, 4, 1) == \
-        256 + 256 + 1024 + 256 + (16 * 2 + 192) * 16 + (16 * 16 + 192) * 16 + 16 * 16 * 4 + 192 * 256 * 256 * 2 + \
-        32 * 8 * 512 * 128 * 4 + 256 * 4 * 4 + 256 * 4 * 4096 * 2 + 2048 * 256 * 2
+        256 + 3 * 512 + 8 * 4 * 16 * 2 * 32768 + 256 * 4 * 4 + 256 * 4 * 4096 * 2 + 2048 * 256 * 2
     assert lib.pmoe_fused_moe_bf16_workspace_bytes(256, 4096, 512, 8, 2048, 4, 0) == \
         lib.pmoe_fused_moe_bf16_workspace_bytes(256, 4096, 512, 8, 2048, 4, 1)
-    # a one-token decode call does not hold the worst case of the tail buffers (88 MB)
-    assert lib.pmoe_fused_moe_bf16_workspace_bytes(1, 4096, 512, 8, 1024, 2, 1) < 64 << 20
+    # no partial sums are reserved for a problem too large for the deep split
+    assert lib.pmoe_fused_moe_bf16_workspace_bytes(4096, 4096, 28672, 8, 9216, 2, 1) == \
+        256 + 3 * 1280 + 8192 * 4 + 8192 * 4096 * 2 + 9216 * 14336 * 2
+    # mxfp8: header (256 B) + row-tile list (8 B per block) + the two work lists (16 B per block and weight tile)
+    # + inverse of the sorted order + y + act (rows * H e4m3) + act scales + re-tiled x scales
     assert lib.pmoe_fused_moe_mxfp8_workspace_bytes(64, 7168, 4096, 256, 33024, 8, 1) == \
-        256 + 256 + 1024 + 2304 + (258 * 16 + 192) * 16 + 118784 + 64 * 8 * 4 + 64 * 8 * 7168 * 2 + 33024 * 2048 + \
+        256 + 2304 + 258 * 16 * 16 + 115712 + 64 * 8 * 4 + 64 * 8 * 7168 * 2 + 33024 * 2048 + \
         33024 * 64 + 33024 * 224
     # rejected before any HIP call: status 1 and a message
     rc = lib.pmoe_moe_align(None, None, None, None, 8, 2000, 128, 128, 1024, 8, None)

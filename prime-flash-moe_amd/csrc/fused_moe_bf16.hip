@@ -15,8 +15,9 @@
 
 namespace pmoe {
 
-// Inclusive scan of one int per thread over a workgroup of 256 threads; `s_part` holds 4 ints.
-__device__ __forceinline__ int block_scan_256(int v, int *s_part) {
+constexpr int kPrologueThreads = 1024;
+// Inclusive scan of one int per thread over the workgroup of the prologue; `s_part` holds an int per wave.
+__device__ __forceinline__ int block_scan(int v, int *s_part) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -54,71 +55,106 @@ __device__ __forceinline__ float estimate_kernel(int n_tiles, int f2, int n_wt, 
     return t;
 }
 
-// Prologue of a bf16 call.  Workgroup 0 builds the row tiles and the plan: runs of blocks with one expert
-// (one pass of block-wide scans per 256 blocks), per run the last row that holds a pair (a thread per run
-// reads the 128 ids of the run's last block), for each kernel the cut into tiles that the cost model likes
-// best and the split of its tail.  All workgroups invert the sorted order: inv[pair id] = sorted row.  Entries
-// of pairs that are not in the schedule keep whatever the buffer held; the reader validates an entry against
-// sorted_ids.
-__global__ __launch_bounds__(256) void moe_tall_prologue_kernel(MoeArgs a, int n_wt_up, int n_wt_down, int n_cus,
+// Prologue of a bf16 call.  Workgroup 0 builds the row tiles and the plan:
+//  1. runs of blocks with one expert (a thread per block, block-wide scans per 1024 blocks); the thread of a run's
+//     last block reads that block's 128 ids for the last row that holds a pair: the run has f2 pairs of fragments;
+//  2. per kernel the cut (fg_max) that the cost model likes best, and the split of its tail;
+//  3. the runs in the order of falling f2 (a counting sort; runs of one size in the order their threads arrive,
+//     which only moves equal tiles in the schedule): the walk of a kernel then ends with the small tiles, and
+//     what is left over when the CUs run out of jobs is short;
+//  4. the tiles of the two cuts.
+// The list of runs lives in LDS (in the workspace when there are more than kLdsRuns blocks).
+// All workgroups invert the sorted order: inv[pair id] = sorted row.  Entries of pairs that are not in the
+// schedule keep whatever the buffer held; the reader validates an entry against sorted_ids.
+constexpr int kLdsRuns = 2048;
+constexpr int kSizeKeys = 128;  // runs are ordered by min(f2, kSizeKeys - 1)
+__global__ __launch_bounds__(kPrologueThreads) void moe_tall_prologue_kernel(MoeArgs a, int n_wt_up, int n_wt_down, int n_cus,
                                                                 int do_invert) {
     const int n_pairs = a.M * a.top_k;
     if (blockIdx.x == 0) {
-        __shared__ int s_part[4], s_carry, s_fg_max[2];
-        __shared__ int s_sum[8];  // per candidate fg_max 6 .. 3: tiles; [4]: pairs of fragments
+        __shared__ int4 s_runs[kLdsRuns];  // {first block, f2, expert, 0}
+        __shared__ int s_order[kLdsRuns];
+        __shared__ int s_part[kPrologueThreads / 64], s_carry[2], s_fg_max[2];
+        __shared__ int s_sum[8];            // per candidate fg_max 6 .. 3: tiles; [4]: pairs of fragments
+        __shared__ int s_hist[kSizeKeys];   // runs per size key, then the first place of each key in the order
         const int tid = threadIdx.x;
         const int n_live = min((a.ntpp[0] + kBlockRows - 1) / kBlockRows, a.n_blocks);
-        // runs of equal expert ids
-        if (tid == 0) s_carry = 0;
+        int4 *runs = n_live <= kLdsRuns ? s_runs : a.runs;
+        int *order = n_live <= kLdsRuns ? s_order : reinterpret_cast<int *>(a.runs + n_live);
+        if (tid < 2) s_carry[tid] = tid == 0 ? -1 : 0;
         if (tid < 8) s_sum[tid] = 0;
-        if (tid < 16) a.plan->counters[tid] = 0;
+        if (tid < kSizeKeys) s_hist[tid] = 0;
+        if (tid < 16) a.plan->counters[tid] = n_cus / 8;  // the first slots are taken without asking (see ask_slot)
         __syncthreads();
-        for (int base = 0; base < n_live; base += 256) {
+        // 1. runs
+        for (int base = 0; base < n_live; base += kPrologueThreads) {
             const int b = base + tid;
             const bool live = b < n_live;
             const int e = live ? a.expert_ids[b] : -1;
             const bool is_start = live && (b == 0 || a.expert_ids[b - 1] != e);
-            const int incl = block_scan_256(is_start ? 1 : 0, s_part);
-            const int carry = s_carry;
-            if (is_start) a.runs[carry + incl - 1] = make_int4(b, 0, 0, 0);
-            __syncthreads();
-            if (tid == 255) s_carry = carry + incl;
-            __syncthreads();
-        }
-        const int n_runs = s_carry;
-        __threadfence_block();
-        __syncthreads();
-        // per run: pairs of fragments up to its last live row; totals per candidate cut
-        int my_tiles[4] = {0, 0, 0, 0}, my_f2 = 0;
-        for (int i = tid; i < n_runs; i += 256) {
-            const int b0 = a.runs[i].x;
-            const int b1 = i + 1 < n_runs ? a.runs[i + 1].x : n_live;
-            const int e = a.expert_ids[b0];
-            int f2 = 0;
-            if (e >= 0 && e < a.E) {
-                const int s0 = (b1 - 1) * kBlockRows;
-                int last = -1;
-                for (int r = 0; r < kBlockRows; ++r) {
-                    const int p = s0 + r < a.sorted_num ? a.sorted_ids[s0 + r] : -1;
-                    if ((unsigned)p < (unsigned)n_pairs) last = r;
+            const bool is_last = live && (b + 1 == n_live || a.expert_ids[b + 1] != e);
+            // start of this block's run: the largest start at or before it
+            int v = is_start ? b : -1;
+            {
+                const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+                for (int d = 1; d < 64; d <<= 1) {
+                    const int t = __shfl_up(v, d, 64);
+                    if (lane >= d) v = max(v, t);
                 }
-                const int rows = (b1 - 1 - b0) * kBlockRows + last + 1;
-                f2 = (rows + 63) >> 6;
+                __syncthreads();
+                if (lane == 63) s_part[wave] = v;
+                __syncthreads();
+                for (int w = 0; w < wave; ++w) v = max(v, s_part[w]);
+                v = max(v, s_carry[0]);
             }
-            a.runs[i].z = f2;
-            my_f2 += f2;
+            const int run_start = v;
+            int f2 = 0;
+            if (is_last && e >= 0 && e < a.E) {
+                const int s0 = b * kBlockRows;
+                int last = -1;
+                if (s0 + kBlockRows <= a.sorted_num && (reinterpret_cast<uintptr_t>(a.sorted_ids) & 15) == 0) {
+                    // all 32 loads in flight together
+                    const int4 *src = reinterpret_cast<const int4 *>(a.sorted_ids + s0);
+                    int4 v[kBlockRows / 4];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) my_tiles[c] += (f2 + 5 - c) / (6 - c);
+                    for (int r = 0; r < kBlockRows / 4; ++r) v[r] = src[r];
+#pragma unroll
+                    for (int r = 0; r < kBlockRows / 4; ++r) {
+                        if ((unsigned)v[r].x < (unsigned)n_pairs) last = 4 * r;
+                        if ((unsigned)v[r].y < (unsigned)n_pairs) last = 4 * r + 1;
+                        if ((unsigned)v[r].z < (unsigned)n_pairs) last = 4 * r + 2;
+                        if ((unsigned)v[r].w < (unsigned)n_pairs) last = 4 * r + 3;
+                    }
+                } else {
+                    for (int r = 0; r < kBlockRows; ++r) {
+                        const int p = s0 + r < a.sorted_num ? a.sorted_ids[s0 + r] : -1;
+                        if ((unsigned)p < (unsigned)n_pairs) last = r;
+                    }
+                }
+                f2 = ((b - run_start) * kBlockRows + last + 1 + 63) >> 6;
+            }
+            const int incl = block_scan(f2 > 0 ? 1 : 0, s_part);
+            const int carry = s_carry[1];
+            if (f2 > 0) {
+                runs[carry + incl - 1] = make_int4(run_start, f2, e, 0);
+                atomicAdd(&s_hist[min(f2, kSizeKeys - 1)], 1);
+                atomicAdd(&s_sum[4], f2);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) atomicAdd(&s_sum[c], (f2 + 5 - c) / (6 - c));
+            }
+            __syncthreads();
+            if (tid == kPrologueThreads - 1) {
+                s_carry[0] = run_start;
+                s_carry[1] = carry + incl;
+            }
+            __syncthreads();
         }
-#pragma unroll
-        for (int c = 0; c < 4; ++c)
-            if (my_tiles[c]) atomicAdd(&s_sum[c], my_tiles[c]);
-        if (my_f2) atomicAdd(&s_sum[4], my_f2);
+        const int n_runs = s_carry[1];
         __threadfence_block();
-        __syncthreads();
+        // 2. the plans: tid 0 the up kernel's, tid 1 the down kernel's: the candidate with the smallest estimate;
+        // one below 6 has to win by 3 % (the model is coarse)
         if (tid < 2) {
-            // tid 0 plans the up kernel, tid 1 the down kernel: the candidate with the smallest estimate; one
-            // below 6 has to win by 3 % (the model is coarse)
             const int n_wt = tid ? n_wt_down : n_wt_up, n_slabs = (tid ? a.H : a.K) * 2 / tall::kRB;
             KernelPlan kp{};
             int best = 6;
@@ -128,7 +164,7 @@ __global__ __launch_bounds__(256) void moe_tall_prologue_kernel(MoeArgs a, int n
                 const float t = estimate_kernel(s_sum[c], s_sum[4], n_wt, n_slabs, n_cus, parts, tail);
                 if (c == 0 || t < 0.97f * best_t) {
                     best = 6 - c;
-                    best_t = c == 0 ? t : t / 0.97f;
+                    best_t = t;
                     kp.n_tiles = s_sum[c];
                     kp.parts = parts;
                     kp.tail = tail;
@@ -149,31 +185,49 @@ __global__ __launch_bounds__(256) void moe_tall_prologue_kernel(MoeArgs a, int n
             }
             s_fg_max[tid] = best;
         }
+        // 3. order of the runs: by falling size key, runs of one key in their own order.  First place of each key ...
+        if (tid < 64) {
+            // (one wave: key k's place = runs with a larger key; two keys per lane, largest keys first)
+            const int k_hi = kSizeKeys - 1 - 2 * tid, k_lo = k_hi - 1;
+            const int c_hi = s_hist[k_hi], c_lo = s_hist[k_lo];
+            int incl = c_hi + c_lo;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int t = __shfl_up(incl, d, 64);
+                if (tid >= d) incl += t;
+            }
+            s_hist[k_hi] = incl - c_hi - c_lo;
+            s_hist[k_lo] = incl - c_lo;
+        }
         __syncthreads();
-        // the tiles of the two cuts (one pass each; the same cut is written twice, into both tables)
-        for (int k = 0; k < 2; ++k) {
+        // ... then every run takes the next place of its key
+        for (int i = tid; i < n_runs; i += kPrologueThreads) order[atomicAdd(&s_hist[min(runs[i].y, kSizeKeys - 1)], 1)] = i;
+        __syncthreads();
+        __threadfence_block();
+        // 4. the tiles of the two cuts (one pass when both kernels use the same cut)
+        const bool same = s_fg_max[0] == s_fg_max[1];
+        for (int k = 0; k < (same ? 1 : 2); ++k) {
             const int fg_max = s_fg_max[k];
-            int4 *tiles = k ? a.tiles_down : a.tiles;
-            if (tid == 0) s_carry = 0;
+            if (tid == 0) s_carry[0] = 0;
             __syncthreads();
-            for (int base = 0; base < n_runs; base += 256) {
+            for (int base = 0; base < n_runs; base += kPrologueThreads) {
                 const int i = base + tid;
-                const int f2 = i < n_runs ? a.runs[i].z : 0;
+                int4 r = make_int4(0, 0, 0, 0);
+                if (i < n_runs) r = runs[order[i]];
+                const int f2 = r.y;
                 const int n = (f2 + fg_max - 1) / fg_max;
-                const int incl = block_scan_256(n, s_part);
-                const int carry = s_carry;
-                if (n > 0) {
-                    const int b0 = a.runs[i].x;
-                    const int e = a.expert_ids[b0];
-                    int t = carry + incl - n, frag = 4 * b0;
-                    for (int q = 0; q < n; ++q) {
-                        const int fg = f2 / n + (q < f2 % n ? 1 : 0);
-                        tiles[t + q] = make_int4(frag, fg, e, 0);
-                        frag += 2 * fg;
-                    }
+                const int incl = block_scan(n, s_part);
+                const int carry = s_carry[0];
+                int t = carry + incl - n, frag = 4 * r.x;
+                for (int q = 0; q < n; ++q) {
+                    const int fg = f2 / n + (q < f2 % n ? 1 : 0);
+                    const int4 tl = make_int4(frag, fg, r.z, 0);
+                    if (k == 0) a.tiles[t + q] = tl;
+                    if (k == 1 || same) a.tiles_down[t + q] = tl;
+                    frag += 2 * fg;
                 }
                 __syncthreads();
-                if (tid == 255) s_carry = carry + incl;
+                if (tid == kPrologueThreads - 1) s_carry[0] = carry + incl;
                 __syncthreads();
             }
         }
@@ -214,14 +268,29 @@ __device__ __forceinline__ float4 *partial_block(const MoeArgs &a, int part, int
            (((int64_t)part * (4 * a.n_blocks) + frag) * a.n_wtiles + wt) * 2048;
 }
 
+// The queue of an XCD: its workgroups (workgroup w is number w / 8 of XCD w mod 8) start with the slot of their own
+// number and take further slots from the XCD's counter, which the prologue sets to the number of workgroups
+// per XCD.  Thread 0 asks for the next slot when the K loop of a tile ends (`ask`), so that the answer arrives
+// under the epilogue (asked earlier, a busy workgroup would hold a job that an idle one could run); `pass`
+// hands it to every thread through `word`, a word of LDS that nothing else uses at that moment.
+__device__ __forceinline__ int ask_slot(int *counter) { return threadIdx.x == 0 ? atomicAdd(counter, 1) : 0; }
+__device__ __forceinline__ int pass_slot(int asked, int *word) {
+    __syncthreads();  // whatever used the LDS before is done
+    if (threadIdx.x == 0) *word = asked;
+    __syncthreads();
+    const int pos = *word;
+    __syncthreads();  // everybody has read the word: the LDS is free again
+    return __builtin_amdgcn_readfirstlane(pos);
+}
+
 // Up kernel tile: token fragments f0 .. f0 + 2 FG - 1 x activation columns [128 wt, 128 wt + 128) of expert e,
 // contraction slabs [slab0, slab0 + n_slabs).  LDS weight rows 0..127 are gate rows, 128..255 the matching up
 // rows; wave v of a group owns gate/up rows 32v..32v+31, so gate and up of one activation element sit in the
 // same lane and register: SwiGLU in registers, the 2H-wide tensor never leaves the chip.
 // deep_part >= 0: the contraction is shared (deep mode); the fp32 sums go to up_partials instead.
 template <int FG>
-__device__ __forceinline__ void up_tile_tall(const MoeArgs &a, int e, int f0, int wt, int slab0, int n_slabs,
-                                             int deep_part, int pos, char *lds) {
+__device__ __forceinline__ int up_tile_tall(const MoeArgs &a, int e, int f0, int wt, int slab0, int n_slabs,
+                                            int deep_part, int pos, int *counter, char *lds) {
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave >> 2, w4 = wave & 3;
     const int K = a.K, H = a.H, N = a.N;
@@ -242,6 +311,7 @@ __device__ __forceinline__ void up_tile_tall(const MoeArgs &a, int e, int f0, in
     zero_acc<FG>(acc);
     const int start = (pos & 7) % n_slabs;  // workgroups that run side by side start their K walks at different slabs
     tall::main_loop<FG>(acc, ld, lds, n_slabs, wrow, grp * FG, lane, start);
+    const int asked = ask_slot(counter);
 
     const int r = lane & 31, half = lane >> 5;
     if (deep_part >= 0) {
@@ -255,7 +325,7 @@ __device__ __forceinline__ void up_tile_tall(const MoeArgs &a, int e, int f0, in
                     dst[((f * 4 + q) * 4 + w4) * 64 + lane] =
                         make_float4(acc[f][t][4 * q], acc[f][t][4 * q + 1], acc[f][t][4 * q + 2], acc[f][t][4 * q + 3]);
         }
-        return;
+        return asked;
     }
     // register i of lane l = activation column 32 w4 + 8(i/4) + 4(l/32) + i%4 of token row 32 t + l%32
     char *tile = lds + grp * (32 * FG * kActPitchBf16);
@@ -282,17 +352,7 @@ __device__ __forceinline__ void up_tile_tall(const MoeArgs &a, int e, int f0, in
         const uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchBf16 + c * 16);
         store_once(a.act + ((grow0 + row) * H + h0) * 2 + c * 16, v);
     }
-}
-
-// Takes the next slot of this workgroup's XCD queue; every thread gets the same number.  `word` is a word of LDS
-// that nothing else uses at this moment.
-__device__ __forceinline__ int next_slot(int *counter, int *word) {
-    __syncthreads();  // whatever used the LDS before is done
-    if (threadIdx.x == 0) *word = atomicAdd(counter, 1);
-    __syncthreads();
-    const int pos = *word;
-    __syncthreads();  // everybody has read the word: the LDS is free again
-    return __builtin_amdgcn_readfirstlane(pos);
+    return asked;
 }
 
 __global__ __launch_bounds__(512) void moe_up_tall_kernel(MoeArgs a) {
@@ -300,12 +360,16 @@ __global__ __launch_bounds__(512) void moe_up_tall_kernel(MoeArgs a) {
     const KernelPlan kp = a.plan->up;
     const int xcd = (int)(blockIdx.x & 7);
     const int n_slabs_all = a.K * 2 / tall::kRB;
-    for (;;) {
-        const int pos = next_slot(&a.plan->counters[xcd], reinterpret_cast<int *>(lds));
+    int *counter = &a.plan->counters[xcd];
+    for (int pos = (int)(blockIdx.x >> 3);;) {
         TallJob j;
         const int st = resolve_tall_job(8 * pos + xcd, a.n_wtiles, kp, j);
         if (st < 0) break;
-        if (st == 0) continue;
+        if (st == 0) {
+            pos = pass_slot(ask_slot(counter), reinterpret_cast<int *>(lds));
+            continue;
+        }
+        int asked = 0;
         const int4 tl = a.tiles[j.tile];
         int f0 = tl.x, fg = tl.y;
         const int e = tl.z;
@@ -319,14 +383,15 @@ __global__ __launch_bounds__(512) void moe_up_tall_kernel(MoeArgs a) {
         }
         fg = __builtin_amdgcn_readfirstlane(fg);
         switch (fg) {
-            case 1: up_tile_tall<1>(a, e, f0, j.wt, slab0, n_slabs, deep_part, pos, lds); break;
-            case 2: up_tile_tall<2>(a, e, f0, j.wt, slab0, n_slabs, deep_part, pos, lds); break;
-            case 3: up_tile_tall<3>(a, e, f0, j.wt, slab0, n_slabs, deep_part, pos, lds); break;
-            case 4: up_tile_tall<4>(a, e, f0, j.wt, slab0, n_slabs, deep_part, pos, lds); break;
-            case 5: up_tile_tall<5>(a, e, f0, j.wt, slab0, n_slabs, deep_part, pos, lds); break;
-            case 6: up_tile_tall<6>(a, e, f0, j.wt, slab0, n_slabs, deep_part, pos, lds); break;
-            default: break;
+            case 1: asked = up_tile_tall<1>(a, e, f0, j.wt, slab0, n_slabs, deep_part, pos, counter, lds); break;
+            case 2: asked = up_tile_tall<2>(a, e, f0, j.wt, slab0, n_slabs, deep_part, pos, counter, lds); break;
+            case 3: asked = up_tile_tall<3>(a, e, f0, j.wt, slab0, n_slabs, deep_part, pos, counter, lds); break;
+            case 4: asked = up_tile_tall<4>(a, e, f0, j.wt, slab0, n_slabs, deep_part, pos, counter, lds); break;
+            case 5: asked = up_tile_tall<5>(a, e, f0, j.wt, slab0, n_slabs, deep_part, pos, counter, lds); break;
+            case 6: asked = up_tile_tall<6>(a, e, f0, j.wt, slab0, n_slabs, deep_part, pos, counter, lds); break;
+            default: asked = ask_slot(counter); break;
         }
+        pos = pass_slot(asked, reinterpret_cast<int *>(lds));
     }
 }
 
@@ -378,7 +443,7 @@ __global__ __launch_bounds__(256) void moe_up_join_kernel(MoeArgs a) {
 // bf16 and transposed through LDS (one group after the other: both do not fit), then all 512 threads store
 // its rows, 512 contiguous bytes each, to y[pair id]; rows without a pair are skipped.
 template <int FG>
-__device__ __forceinline__ void down_tile_tall(const MoeArgs &a, int e, int f0, int wt, int pos, char *lds) {
+__device__ __forceinline__ int down_tile_tall(const MoeArgs &a, int e, int f0, int wt, int pos, int *counter, char *lds) {
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave >> 2, w4 = wave & 3;
     const int K = a.K, H = a.H;
@@ -397,6 +462,7 @@ __device__ __forceinline__ void down_tile_tall(const MoeArgs &a, int e, int f0, 
     zero_acc<FG>(acc);
     const int start = (pos & 7) % n_slabs;  // workgroups that run side by side start their K walks at different slabs
     tall::main_loop<FG>(acc, ld, lds, n_slabs, wrow, grp * FG, lane, start);
+    const int asked = ask_slot(counter);
 
     const int r = lane & 31, half = lane >> 5;
     const int cols = min(kWRows, K - k0);
@@ -441,32 +507,38 @@ __device__ __forceinline__ void down_tile_tall(const MoeArgs &a, int e, int f0, 
         }
         if (g == 0) __syncthreads();
     }
+    return asked;
 }
 
 __global__ __launch_bounds__(512) void moe_down_tall_kernel(MoeArgs a) {
     __shared__ __attribute__((aligned(1024))) char lds[tall::kLdsBytes];
     const KernelPlan kp = a.plan->down;
     const int xcd = (int)(blockIdx.x & 7);
-    for (;;) {
-        const int pos = next_slot(&a.plan->counters[8 + xcd], reinterpret_cast<int *>(lds));
+    int *counter = &a.plan->counters[8 + xcd];
+    for (int pos = (int)(blockIdx.x >> 3);;) {
         TallJob j;
         const int st = resolve_tall_job(8 * pos + xcd, a.n_wtiles, kp, j);
         if (st < 0) break;
-        if (st == 0) continue;
+        if (st == 0) {
+            pos = pass_slot(ask_slot(counter), reinterpret_cast<int *>(lds));
+            continue;
+        }
+        int asked = 0;
         const int4 tl = a.tiles_down[j.tile];
         int f0 = tl.x, fg = tl.y;
         const int e = tl.z;
         if (j.parts > 1) fg = row_split(f0, fg, j.part, j.parts);
         fg = __builtin_amdgcn_readfirstlane(fg);
         switch (fg) {
-            case 1: down_tile_tall<1>(a, e, f0, j.wt, pos, lds); break;
-            case 2: down_tile_tall<2>(a, e, f0, j.wt, pos, lds); break;
-            case 3: down_tile_tall<3>(a, e, f0, j.wt, pos, lds); break;
-            case 4: down_tile_tall<4>(a, e, f0, j.wt, pos, lds); break;
-            case 5: down_tile_tall<5>(a, e, f0, j.wt, pos, lds); break;
-            case 6: down_tile_tall<6>(a, e, f0, j.wt, pos, lds); break;
-            default: break;
+            case 1: asked = down_tile_tall<1>(a, e, f0, j.wt, pos, counter, lds); break;
+            case 2: asked = down_tile_tall<2>(a, e, f0, j.wt, pos, counter, lds); break;
+            case 3: asked = down_tile_tall<3>(a, e, f0, j.wt, pos, counter, lds); break;
+            case 4: asked = down_tile_tall<4>(a, e, f0, j.wt, pos, counter, lds); break;
+            case 5: asked = down_tile_tall<5>(a, e, f0, j.wt, pos, counter, lds); break;
+            case 6: asked = down_tile_tall<6>(a, e, f0, j.wt, pos, counter, lds); break;
+            default: asked = ask_slot(counter); break;
         }
+        pos = pass_slot(asked, reinterpret_cast<int *>(lds));
     }
 }
 
@@ -484,7 +556,8 @@ size_t bf16_workspace(MoeArgs &a, char *ws) {
         return ws != nullptr ? ws + at : nullptr;
     };
     a.plan = reinterpret_cast<TallPlan *>(take(sizeof(TallPlan)));
-    a.runs = reinterpret_cast<int4 *>(take((blocks + 1) * sizeof(int4)));
+    // (run list and its order, used when they do not fit the LDS of the prologue)
+    a.runs = reinterpret_cast<int4 *>(take((blocks + 1) * (sizeof(int4) + sizeof(int))));
     // a cut has at most ceil(f2 / 3) tiles per expert, f2 <= 2 blocks of its expert
     a.tiles = reinterpret_cast<int4 *>(take((blocks + 1) * sizeof(int4)));
     a.tiles_down = reinterpret_cast<int4 *>(take((blocks + 1) * sizeof(int4)));
@@ -507,8 +580,8 @@ int launch_bf16_pipeline(MoeArgs a, void *out, int split, hipStream_t s) {
     {
         // the plan is needed by the two kernels even when the rest of the prologue is masked off
         const int do_invert = (mask & PMOE_PHASE_PROLOGUE) ? 1 : 0;
-        const int blocks = do_invert ? std::max(1, std::min((a.sorted_num + 255) / 256, 1024)) : 1;
-        hipLaunchKernelGGL(moe_tall_prologue_kernel, dim3(blocks), dim3(256), 0, s, a, n_wt_up, n_wt_down, n_cus,
+        const int blocks = do_invert ? std::max(1, std::min((a.sorted_num + kPrologueThreads - 1) / kPrologueThreads, 512)) : 1;
+        hipLaunchKernelGGL(moe_tall_prologue_kernel, dim3(blocks), dim3(kPrologueThreads), 0, s, a, n_wt_up, n_wt_down, n_cus,
                            do_invert);
     }
     if (a.n_blocks > 0) {

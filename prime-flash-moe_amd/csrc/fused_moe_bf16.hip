@@ -34,7 +34,9 @@ __device__ __forceinline__ int block_scan(int v, int *s_part) {
 // Estimated time of a kernel (in units of a third of a microsecond) whose `f2` pairs of fragments are cut into
 // `n_tiles` row tiles: whole rounds of the chip's CUs at the cost of a mean tile, plus a last round whose jobs
 // are shared by rows.  A tile of g pairs costs (0.6 + g) per slab of its K loop (measured: 0.18 + 0.34 g us on
-// tiles of 2 to 6 pairs) and 3 + 2.5 g for set-up and epilogue.
+// tiles of 2 to 6 pairs) and 3 + 2.5 g for set-up and epilogue; a round of nothing but shared jobs costs 1.3
+// times what its small tiles would among large ones (measured on the Mixtral-like down kernel: every weight row
+// is then read twice as often).
 __device__ __forceinline__ float estimate_kernel(int n_tiles, int f2, int n_wt, int n_slabs, int n_cus, int &parts,
                                                  int &tail) {
     parts = 1;
@@ -45,8 +47,8 @@ __device__ __forceinline__ float estimate_kernel(int n_tiles, int f2, int n_wt, 
     const int jobs = n_tiles * n_wt, rounds = jobs / n_cus, rest = jobs % n_cus;
     float t = (float)rounds * cost(g);
     if (rest > 0) {
-        int p = rounds >= 16 ? 1 : min(min(4, n_cus / rest), max(1, (int)g));
-        t += cost(g / (float)p);
+        const int p = rounds >= 16 ? 1 : min(min(4, n_cus / rest), max(1, (int)g));
+        t += p > 1 ? 1.3f * cost(g / (float)p) : cost(g);
         if (p > 1) {
             parts = p;
             tail = rest;
@@ -54,15 +56,35 @@ __device__ __forceinline__ float estimate_kernel(int n_tiles, int f2, int n_wt, 
     }
     return t;
 }
+// Number of row tiles for a kernel with n_wt weight tiles: the fewest there can be (t_min, tiles of up to 6
+// pairs), or, if the estimate likes it better, the next number that fills whole rounds of the CUs (smaller
+// tiles, nothing left over), as long as that is at most half as many again and fits the tables (t_cap).
+__device__ __forceinline__ int choose_tiles(int t_min, int t_cap, int f2, int n_wt, int n_slabs, int n_cus) {
+    if (t_min <= 0) return 0;
+    int g = n_cus, r = n_wt;  // gcd
+    while (r) {
+        const int x = g % r;
+        g = r;
+        r = x;
+    }
+    const int step = n_cus / g;  // tiles x n_wt is a multiple of n_cus for every multiple of step
+    const int t_full = (t_min + step - 1) / step * step;
+    if (t_full == t_min || t_full > t_cap || 2 * t_full > 3 * t_min || t_full > f2) return t_min;
+    int parts, tail;
+    const float e_min = estimate_kernel(t_min, f2, n_wt, n_slabs, n_cus, parts, tail);
+    const float e_full = estimate_kernel(t_full, f2, n_wt, n_slabs, n_cus, parts, tail);
+    return e_full < 0.98f * e_min ? t_full : t_min;
+}
 
 // Prologue of a bf16 call.  Workgroup 0 builds the row tiles and the plan:
 //  1. runs of blocks with one expert (a thread per block, block-wide scans per 1024 blocks); the thread of a run's
 //     last block reads that block's 128 ids for the last row that holds a pair: the run has f2 pairs of fragments;
-//  2. per kernel the cut (fg_max) that the cost model likes best, and the split of its tail;
+//  2. per kernel the number of row tiles (see choose_tiles);
 //  3. the runs in the order of falling f2 (a counting sort; runs of one size in the order their threads arrive,
 //     which only moves equal tiles in the schedule): the walk of a kernel then ends with the small tiles, and
 //     what is left over when the CUs run out of jobs is short;
-//  4. the tiles of the two cuts.
+//  4. the tiles of the two cuts (a run gets the tiles it needs at 6 pairs a tile, and the largest runs one more
+//     each until the chosen number is reached), then the plans with the split of the tails.
 // The list of runs lives in LDS (in the workspace when there are more than kLdsRuns blocks).
 // All workgroups invert the sorted order: inv[pair id] = sorted row.  Entries of pairs that are not in the
 // schedule keep whatever the buffer held; the reader validates an entry against sorted_ids.
@@ -74,8 +96,8 @@ __global__ __launch_bounds__(kPrologueThreads) void moe_tall_prologue_kernel(Moe
     if (blockIdx.x == 0) {
         __shared__ int4 s_runs[kLdsRuns];  // {first block, f2, expert, 0}
         __shared__ int s_order[kLdsRuns];
-        __shared__ int s_part[kPrologueThreads / 64], s_carry[2], s_fg_max[2];
-        __shared__ int s_sum[8];            // per candidate fg_max 6 .. 3: tiles; [4]: pairs of fragments
+        __shared__ int s_part[kPrologueThreads / 64], s_carry[2], s_want[2], s_tiles[2];
+        __shared__ int s_sum[8];            // [0]: tiles of up to 6 pairs the runs need; [4]: pairs of fragments
         __shared__ int s_hist[kSizeKeys];   // runs per size key, then the first place of each key in the order
         const int tid = threadIdx.x;
         const int n_live = min((a.ntpp[0] + kBlockRows - 1) / kBlockRows, a.n_blocks);
@@ -140,8 +162,7 @@ __global__ __launch_bounds__(kPrologueThreads) void moe_tall_prologue_kernel(Moe
                 runs[carry + incl - 1] = make_int4(run_start, f2, e, 0);
                 atomicAdd(&s_hist[min(f2, kSizeKeys - 1)], 1);
                 atomicAdd(&s_sum[4], f2);
-#pragma unroll
-                for (int c = 0; c < 4; ++c) atomicAdd(&s_sum[c], (f2 + 5 - c) / (6 - c));
+                atomicAdd(&s_sum[0], (f2 + 5) / 6);
             }
             __syncthreads();
             if (tid == kPrologueThreads - 1) {
@@ -152,38 +173,10 @@ __global__ __launch_bounds__(kPrologueThreads) void moe_tall_prologue_kernel(Moe
         }
         const int n_runs = s_carry[1];
         __threadfence_block();
-        // 2. the plans: tid 0 the up kernel's, tid 1 the down kernel's: the candidate with the smallest estimate;
-        // one below 6 has to win by 3 % (the model is coarse)
+        // 2. the number of row tiles of each kernel: tid 0 the up kernel's, tid 1 the down kernel's
         if (tid < 2) {
             const int n_wt = tid ? n_wt_down : n_wt_up, n_slabs = (tid ? a.H : a.K) * 2 / tall::kRB;
-            KernelPlan kp{};
-            int best = 6;
-            float best_t = 0.f;
-            for (int c = 0; c < 4; ++c) {
-                int parts, tail;
-                const float t = estimate_kernel(s_sum[c], s_sum[4], n_wt, n_slabs, n_cus, parts, tail);
-                if (c == 0 || t < 0.97f * best_t) {
-                    best = 6 - c;
-                    best_t = t;
-                    kp.n_tiles = s_sum[c];
-                    kp.parts = parts;
-                    kp.tail = tail;
-                }
-            }
-            if (tid == 0) {
-                const int jobs_up = kp.n_tiles * n_wt_up, up_slabs = a.K * 2 / tall::kRB;
-                int deep_parts = 1;
-                if (a.deep_ok && jobs_up > 0) deep_parts = min(min(kDeepParts, up_slabs / 4), n_cus / jobs_up);
-                if (deep_parts >= 2) {
-                    kp.deep = 1;
-                    kp.parts = deep_parts;
-                    kp.tail = 0;
-                }
-                a.plan->up = kp;
-            } else {
-                a.plan->down = kp;
-            }
-            s_fg_max[tid] = best;
+            s_want[tid] = choose_tiles(s_sum[0], a.n_blocks, s_sum[4], n_wt, n_slabs, n_cus);
         }
         // 3. order of the runs: by falling size key, runs of one key in their own order.  First place of each key ...
         if (tid < 64) {
@@ -204,18 +197,20 @@ __global__ __launch_bounds__(kPrologueThreads) void moe_tall_prologue_kernel(Moe
         for (int i = tid; i < n_runs; i += kPrologueThreads) order[atomicAdd(&s_hist[min(runs[i].y, kSizeKeys - 1)], 1)] = i;
         __syncthreads();
         __threadfence_block();
-        // 4. the tiles of the two cuts (one pass when both kernels use the same cut)
-        const bool same = s_fg_max[0] == s_fg_max[1];
+        // 4. the tiles of the two cuts (one pass when both kernels use the same cut), and the plans
+        const int t_min = s_sum[0];
+        const bool same = s_want[0] == s_want[1];
         for (int k = 0; k < (same ? 1 : 2); ++k) {
-            const int fg_max = s_fg_max[k];
+            const int extra = max(s_want[k] - t_min, 0);
             if (tid == 0) s_carry[0] = 0;
             __syncthreads();
             for (int base = 0; base < n_runs; base += kPrologueThreads) {
-                const int i = base + tid;
+                const int i = base + tid;  // place in the order: the largest runs come first
                 int4 r = make_int4(0, 0, 0, 0);
                 if (i < n_runs) r = runs[order[i]];
                 const int f2 = r.y;
-                const int n = (f2 + fg_max - 1) / fg_max;
+                int n = (f2 + 5) / 6;
+                if (i < n_runs) n = min(f2, n + extra / n_runs + (i < extra % n_runs ? 1 : 0));
                 const int incl = block_scan(n, s_part);
                 const int carry = s_carry[0];
                 int t = carry + incl - n, frag = 4 * r.x;
@@ -229,6 +224,28 @@ __global__ __launch_bounds__(kPrologueThreads) void moe_tall_prologue_kernel(Moe
                 __syncthreads();
                 if (tid == kPrologueThreads - 1) s_carry[0] = carry + incl;
                 __syncthreads();
+            }
+            if (tid == 0) s_tiles[k] = s_carry[0];
+            if (tid == 0 && same) s_tiles[1] = s_carry[0];
+            __syncthreads();
+        }
+        if (tid < 2) {
+            const int n_wt = tid ? n_wt_down : n_wt_up, n_slabs = (tid ? a.H : a.K) * 2 / tall::kRB;
+            KernelPlan kp{};
+            kp.n_tiles = s_tiles[tid];
+            estimate_kernel(kp.n_tiles, s_sum[4], n_wt, n_slabs, n_cus, kp.parts, kp.tail);
+            if (tid == 0) {
+                const int jobs_up = kp.n_tiles * n_wt_up;
+                int deep_parts = 1;
+                if (a.deep_ok && jobs_up > 0) deep_parts = min(min(kDeepParts, n_slabs / 4), n_cus / jobs_up);
+                if (deep_parts >= 2) {
+                    kp.deep = 1;
+                    kp.parts = deep_parts;
+                    kp.tail = 0;
+                }
+                a.plan->up = kp;
+            } else {
+                a.plan->down = kp;
             }
         }
     }
@@ -558,7 +575,7 @@ size_t bf16_workspace(MoeArgs &a, char *ws) {
     a.plan = reinterpret_cast<TallPlan *>(take(sizeof(TallPlan)));
     // (run list and its order, used when they do not fit the LDS of the prologue)
     a.runs = reinterpret_cast<int4 *>(take((blocks + 1) * (sizeof(int4) + sizeof(int))));
-    // a cut has at most ceil(f2 / 3) tiles per expert, f2 <= 2 blocks of its expert
+    // (a cut has at most one tile per block: choose_tiles)
     a.tiles = reinterpret_cast<int4 *>(take((blocks + 1) * sizeof(int4)));
     a.tiles_down = reinterpret_cast<int4 *>(take((blocks + 1) * sizeof(int4)));
     // few up jobs for the chip and a contraction long enough to share: deep mode may be planned

@@ -12,10 +12,11 @@ namespace pmoe {
 //
 // Row tiles: an expert's live rows are F2 pairs of fragments of 32 sorted rows (the rows of its blocks up to
 // the last one that holds a pair, rounded up inside the expert's own padding); they are cut into
-// ceil(F2 / fg_max) tiles of FG pairs each (FG = 1 .. fg_max <= 6, sizes differ by at most one pair).
-// tiles[i] = {first fragment, FG, expert, 0}.  Each of the two kernels has its own cut (its own fg_max, chosen
-// by a cost model so that its jobs fill whole rounds of the chip's CUs): the activation is indexed by sorted
-// row, so the kernels need not agree on the tiles.
+// tiles of FG pairs each (FG = 1 .. 6, the tiles of one expert differ by at most one pair).
+// tiles[i] = {first fragment, FG, expert, 0}.  Each of the two kernels has its own cut: the fewest tiles there
+// can be, or as many more as make its jobs fill whole rounds of the chip's CUs when a cost model prefers that
+// (the largest experts are then cut into one more tile each): the activation is indexed by sorted row, so the
+// kernels need not agree on the tiles.
 //
 // Jobs of a kernel: (row tile, weight tile), n_tiles x n_wt of them, walked in the order
 // [group of 8 weight tiles][row tile][weight tile in group].  The kernels are resident: one workgroup per CU,

@@ -98,16 +98,39 @@ def time_events(step, steps):
     return sum(ms) / len(ms) * 1e-3, ms[len(ms) // 2] * 1e-3
 
 
-def phase_time(step, mask, steps):
+def phase_time(step, mask, steps, inner=1):
+    """Duration of the kernels that `mask` leaves of one call, from replays of a HIP graph captured under that mask
+    (the mask acts when the kernels are enqueued, that is at capture): the time of the kernels themselves, without
+    the host's launch path, which at a few tens of microseconds per call would drown the small shapes."""
     from prime_moe import _native
     lib = _native.load()
     lib.pmoe_set_phase_mask(mask)
     try:
-        for _ in range(2):
-            step()
-        return time_events(step, steps)[0]
+        return graph_time(step, steps, inner)
     finally:
         lib.pmoe_set_phase_mask(PHASE_ALL)
+
+
+def graph_time(step, replays=20, inner=1):
+    """Median duration of `step` in a replayed HIP graph (the reference benchmark's method,
+    benchmark/benchmark.py:355-386): what the call costs without the host's launch path.  `inner` calls are
+    captured back to back in one graph, so that replays of very short calls measure the GPU and not the launch of
+    the graph."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(inner):
+            step()
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    return time_events(graph.replay, replays)[1] / inner
 
 
 def recorded_traffic(config: str, kernel: str = "moe_up_kernel"):
@@ -209,9 +232,13 @@ def run_config(cfg, split, steps, warmup, device, with_cpu, log):
     step = make_step(cfg, inp, sched, out, split)
     sec = time_steps(step, steps, warmup)
     ev_mean, ev_med = time_events(step, steps)
-    # (each of the two includes the prologue's list building, about 10 us, which runs whatever the mask)
-    t_up = phase_time(step, PHASE_UP, steps)
-    t_down = phase_time(step, PHASE_DOWN, steps)
+    # the part of the prologue that builds the schedule runs whatever the mask: it is timed alone and taken off
+    # the two kernels' times, so that they are the kernels' own
+    inner = 8 if sec < 200e-6 else 1
+    t_plan = phase_time(step, 0, steps, inner)
+    t_up = max(phase_time(step, PHASE_UP, steps, inner) - t_plan, 1e-9)
+    t_down = max(phase_time(step, PHASE_DOWN, steps, inner) - t_plan, 1e-9)
+    t_graph = graph_time(step, steps, inner)
     step()
     torch.cuda.synchronize()
     P = cfg.T * cfg.top_k
@@ -221,7 +248,7 @@ def run_config(cfg, split, steps, warmup, device, with_cpu, log):
     peak = PEAK_TFLOPS[cfg.dtype]
     res = {
         "name": cfg.name, "split": bool(split), "sec": sec, "ev_mean": ev_mean, "ev_med": ev_med,
-        "t_up": t_up, "t_down": t_down, "tflops": cfg.flops / sec / 1e12,
+        "t_up": t_up, "t_down": t_down, "t_graph": t_graph, "tflops": cfg.flops / sec / 1e12,
         "pct_mfma": 100 * cfg.flops / sec / 1e12 / peak, "weight_gbs": wb / sec / 1e9,
         "pct_hbm": 100 * total_b / sec / 1e9 / PEAK_HBM_GBS, "weight_bytes": wb, "bytes": total_b,
         "up_tflops": flops_up / t_up / 1e12 if t_up else 0.0,
@@ -230,7 +257,7 @@ def run_config(cfg, split, steps, warmup, device, with_cpu, log):
     log(f"{cfg.name:18s} split={int(split)}  {sec * 1e6:10.1f} us/call  {res['tflops']:8.1f} TFLOP/s "
         f"({res['pct_mfma']:5.1f}% {cfg.dtype} MFMA peak)  weights {res['weight_gbs']:7.1f} GB/s  "
         f"all-bytes {res['pct_hbm']:5.1f}% of 8 TB/s | up {t_up * 1e6:9.1f} us ({res['up_tflops']:7.1f} TF) "
-        f"down {t_down * 1e6:9.1f} us ({res['down_tflops']:7.1f} TF)")
+        f"down {t_down * 1e6:9.1f} us ({res['down_tflops']:7.1f} TF) | graph replay {t_graph * 1e6:9.1f} us")
     # algorithmic bytes of one launch of each kernel: weights (+ scales) of the touched experts once, the routed
     # rows of the token-side operand once, the output written once
     sx = 2 if cfg.dtype == "bf16" else 33 / 32
@@ -278,6 +305,7 @@ def summary(r):
     return {"config": r["name"], "split": r["split"], "us_per_call": round(r["sec"] * 1e6, 1),
             "tflops": round(r["tflops"], 1), "pct_mfma_peak": round(r["pct_mfma"], 2),
             "weight_gbs": round(r["weight_gbs"], 1), "pct_hbm_all_bytes": round(r["pct_hbm"], 2),
+            "graph_us_per_call": round(r["t_graph"] * 1e6, 1),
             "up_kernel_us": round(r["t_up"] * 1e6, 1), "down_kernel_us": round(r["t_down"] * 1e6, 1),
             "other_us": round((r["ev_mean"] - r["t_up"] - r["t_down"]) * 1e6, 1)}
 
@@ -349,7 +377,7 @@ def main():
             for split in ((1, 0) if name.startswith(("c2", "c5")) else (1,)):
                 if name == args.config and split == args.split:
                     continue
-                everything.append(summary(run_config(cfg, split, max(5, args.steps // 2), 5, device, False, log)))
+                everything.append(summary(run_config(cfg, split, args.steps, args.warmup, device, False, log)))
                 torch.cuda.empty_cache()
         router = router_times(device, 20)
         log(f"router front-end on {router['workload']}: fused {router['fused_us']:.1f} us, "
@@ -380,6 +408,13 @@ def main():
     roofline["traffic_source"] = ("profiles/kernel_figures.txt (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier run of "
                                   "this workload, prime_moe/profiling.py)") if traffic is not None else None
     roofline["mfma_busy_recorded"] = mfma_busy
+    # the per-configuration table once more as flat keys (config.<name>.split<0|1>.<figure>), for readers that keep
+    # only the scalar members of `config`
+    flat = {}
+    for e in everything:
+        for k, v in e.items():
+            if k not in ("config", "split"):
+                flat[f"{e['config']}.split{int(e['split'])}.{k}"] = v
     line = {
         "metric": "Fused-MoE TFLOP/s & % MFMA peak (bf16/mxfp8); decode-shape HBM GB/s",
         "value": r["weight_gbs"] if memory_bound else r["tflops"],
@@ -391,7 +426,7 @@ def main():
                                f"block_m=128 split={bool(args.split)}",
                    "flops_per_step": cfg.flops, "pct_mfma_peak": r["pct_mfma"],
                    "weight_gbs": r["weight_gbs"], "parity_rel_clamp_1": r["parity"],
-                   "all": everything, "router": router},
+                   **flat, "all": everything, "router": router},
         "roofline": roofline,
         "cpu_baseline": r["cpu"],
     }

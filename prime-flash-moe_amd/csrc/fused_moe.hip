@@ -195,31 +195,21 @@ __device__ __forceinline__ void swiglu_epilogue(const f32x16 (&acc)[2][4], char 
 #pragma unroll
             for (int i = 0; i < 16; ++i) v[i] = swiglu(acc[0][t][i], acc[1][t][i]);
             const int row = 32 * t + r;
-            if constexpr (DT == DT_BF16) {
+            static_assert(DT == DT_FP8, "the bf16 epilogue lives in fused_moe_bf16.hip");
+            float amax = 0.f;
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int hl = 32 * w4 + 8 * g + 4 * half;  // tile-local activation column
-                    uint2 pk;
-                    pk.x = pack2_bf16(v[4 * g], v[4 * g + 1]);
-                    pk.y = pack2_bf16(v[4 * g + 2], v[4 * g + 3]);
-                    *reinterpret_cast<uint2 *>(tile + row * kActPitchBf16 + hl * 2) = pk;
-                }
-            } else {
-                float amax = 0.f;
+            for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(v[i]));
+            amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+            uint32_t e8;
+            float inv;
+            mx_block_scale(amax, e8, inv);
 #pragma unroll
-                for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(v[i]));
-                amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-                uint32_t e8;
-                float inv;
-                mx_block_scale(amax, e8, inv);
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int hl = 32 * w4 + 8 * g + 4 * half;
-                    const uint32_t q = pack4_e4m3(v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3], inv);
-                    *reinterpret_cast<uint32_t *>(tile + row * kActPitchFp8 + hl) = q;
-                }
-                if (half == 0) reinterpret_cast<uint8_t *>(sc_tile)[row * 4 + w4] = (uint8_t)e8;
+            for (int g = 0; g < 4; ++g) {
+                const int hl = 32 * w4 + 8 * g + 4 * half;
+                const uint32_t q = pack4_e4m3(v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3], inv);
+                *reinterpret_cast<uint32_t *>(tile + row * kActPitchFp8 + hl) = q;
             }
+            if (half == 0) reinterpret_cast<uint8_t *>(sc_tile)[row * 4 + w4] = (uint8_t)e8;
         }
     }
 }
@@ -230,29 +220,18 @@ template <int DT>
 __device__ __forceinline__ void store_act_tile(const MoeArgs &a, const char *tile, const uint32_t *sc_tile,
                                                int64_t row0, int h0, int ntf, int gt) {
     const int H = a.H;
-    if constexpr (DT == DT_BF16) {
-        const int c = gt & 15;
+    static_assert(DT == DT_FP8, "the bf16 epilogue lives in fused_moe_bf16.hip");
+    const int c = gt & 7;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int row = (gt >> 4) + 16 * i;
-            if (row < 32 * ntf) {
-                uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchBf16 + c * 16);
-                store_once(a.act + ((row0 + row) * H + h0) * 2 + c * 16, v);
-            }
+    for (int i = 0; i < 4; ++i) {
+        const int row = (gt >> 3) + 32 * i;
+        if (i < ntf) {
+            uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchFp8 + c * 16);
+            store_once(a.act + (row0 + row) * H + h0 + c * 16, v);
         }
-    } else {
-        const int c = gt & 7;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int row = (gt >> 3) + 32 * i;
-            if (i < ntf) {
-                uint4 v = *reinterpret_cast<const uint4 *>(tile + row * kActPitchFp8 + c * 16);
-                store_once(a.act + (row0 + row) * H + h0 + c * 16, v);
-            }
-        }
-        if (gt < 32 * ntf)
-            a.act_scales[((row0 >> 7) * (H >> 7) + (h0 >> 7)) * kBlockRows + gt] = sc_tile[gt];
     }
+    if (gt < 32 * ntf)
+        a.act_scales[((row0 >> 7) * (H >> 7) + (h0 >> 7)) * kBlockRows + gt] = sc_tile[gt];
 }
 
 // ==========================================================================================
@@ -343,7 +322,7 @@ __device__ __forceinline__ int slab_rotation(int n_slabs) {
 template <int DT, int RB, int NTF>
 __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, const Job &job, RowInfo<2> &ri, char *lds,
                                              uint32_t *act_sc_lds) {
-    constexpr int ES = DT == DT_BF16 ? 2 : 1;
+    constexpr int ES = 1;  // bytes per element
     const int first = job.first, ht = job.wt, n_sub = job.n_sub, e = job.e;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;
@@ -374,7 +353,7 @@ __device__ __forceinline__ void up_tile_ring(const MoeArgs &a, const Job &job, R
     const int start = slab_rotation<RB>(n_slabs);
     const int tok_region = grp ? lay.group1_off : 0;
     // the ring is free after main_loop (it ends with a barrier): its head holds the activation tiles
-    constexpr int kPitch = DT == DT_BF16 ? kActPitchBf16 : kActPitchFp8;
+    constexpr int kPitch = kActPitchFp8;
     char *tile = lds + grp * (kBlockRows * kPitch);
     uint32_t *sc_tile = act_sc_lds + grp * kBlockRows;
     const int SB = lay.stage_bytes, NS = lay.stages;
@@ -420,7 +399,7 @@ struct SplitLds {
     static_assert(sizeof(RowInfo<2>) <= kRowInfoBytes, "row table does not fit its slot");
     // the epilogues reuse the head of the ring: two y tiles (down kernel) or two activation tiles (up kernel)
     static_assert(2 * kBlockRows * kYPitch <= kRing, "y tiles of the epilogue overrun their LDS");
-    static_assert(2 * kBlockRows * kActPitchBf16 <= kRing, "activation tiles of the epilogue overrun the ring");
+    static_assert(2 * kBlockRows * kActPitchFp8 <= kRing, "activation tiles of the epilogue overrun the ring");
 };
 
 template <int DT>
@@ -443,7 +422,7 @@ __global__ __launch_bounds__(512) void moe_up_kernel(MoeArgs a) {
 // routing weights are applied later, by finalize_kernel.
 template <int DT, int RB, int NTF>
 __device__ __forceinline__ void down_tile_ring(const MoeArgs &a, const Job &job, RowInfo<2> &ri, char *lds) {
-    constexpr int ES = DT == DT_BF16 ? 2 : 1;
+    constexpr int ES = 1;  // bytes per element
     const int first = job.first, kt = job.wt, n_sub = job.n_sub, e = job.e;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave >> 2, w4 = wave & 3, gt = tid & 255;

@@ -90,7 +90,7 @@ __device__ __forceinline__ int choose_tiles(int t_min, int t_cap, int f2, int n_
 // schedule keep whatever the buffer held; the reader validates an entry against sorted_ids.
 constexpr int kLdsRuns = 2048;
 constexpr int kSizeKeys = 128;  // runs are ordered by min(f2, kSizeKeys - 1)
-__global__ __launch_bounds__(kPrologueThreads) void moe_tall_prologue_kernel(MoeArgs a, int n_wt_up, int n_wt_down, int n_cus,
+__global__ __launch_bounds__(kPrologueThreads) void moe_prologue_kernel_bf16(MoeArgs a, int n_wt_up, int n_wt_down, int n_cus,
                                                                 int do_invert) {
     const int n_pairs = a.M * a.top_k;
     if (blockIdx.x == 0) {
@@ -372,7 +372,7 @@ __device__ __forceinline__ int up_tile_tall(const MoeArgs &a, int e, int f0, int
     return asked;
 }
 
-__global__ __launch_bounds__(512) void moe_up_tall_kernel(MoeArgs a) {
+__global__ __launch_bounds__(512) void moe_up_kernel_bf16(MoeArgs a) {
     __shared__ __attribute__((aligned(1024))) char lds[tall::kLdsBytes];
     const KernelPlan kp = a.plan->up;
     const int xcd = (int)(blockIdx.x & 7);
@@ -527,7 +527,7 @@ __device__ __forceinline__ int down_tile_tall(const MoeArgs &a, int e, int f0, i
     return asked;
 }
 
-__global__ __launch_bounds__(512) void moe_down_tall_kernel(MoeArgs a) {
+__global__ __launch_bounds__(512) void moe_down_kernel_bf16(MoeArgs a) {
     __shared__ __attribute__((aligned(1024))) char lds[tall::kLdsBytes];
     const KernelPlan kp = a.plan->down;
     const int xcd = (int)(blockIdx.x & 7);
@@ -598,20 +598,20 @@ int launch_bf16_pipeline(MoeArgs a, void *out, int split, hipStream_t s) {
         // the plan is needed by the two kernels even when the rest of the prologue is masked off
         const int do_invert = (mask & PMOE_PHASE_PROLOGUE) ? 1 : 0;
         const int blocks = do_invert ? std::max(1, std::min((a.sorted_num + kPrologueThreads - 1) / kPrologueThreads, 512)) : 1;
-        hipLaunchKernelGGL(moe_tall_prologue_kernel, dim3(blocks), dim3(kPrologueThreads), 0, s, a, n_wt_up, n_wt_down, n_cus,
+        hipLaunchKernelGGL(moe_prologue_kernel_bf16, dim3(blocks), dim3(kPrologueThreads), 0, s, a, n_wt_up, n_wt_down, n_cus,
                            do_invert);
     }
     if (a.n_blocks > 0) {
         // resident kernels: a workgroup per CU (their 160 KB of LDS leave room for one)
         a.n_wtiles = n_wt_up;
         if (mask & PMOE_PHASE_UP) {
-            hipLaunchKernelGGL(moe_up_tall_kernel, dim3(n_cus), dim3(512), 0, s, a);
+            hipLaunchKernelGGL(moe_up_kernel_bf16, dim3(n_cus), dim3(512), 0, s, a);
             if (a.deep_ok)
                 hipLaunchKernelGGL(moe_up_join_kernel, dim3(a.n_blocks * tall::kMaxFrags * n_wt_up * 4), dim3(256), 0, s, a);
         }
         MoeArgs d = a;
         d.n_wtiles = n_wt_down;
-        if (mask & PMOE_PHASE_DOWN) hipLaunchKernelGGL(moe_down_tall_kernel, dim3(n_cus), dim3(512), 0, s, d);
+        if (mask & PMOE_PHASE_DOWN) hipLaunchKernelGGL(moe_down_kernel_bf16, dim3(n_cus), dim3(512), 0, s, d);
     }
     if (mask & PMOE_PHASE_FINALIZE) launch_finalize(a, out, split, n_wt_down, s);
     return check_launch("fused_moe_bf16 launch");

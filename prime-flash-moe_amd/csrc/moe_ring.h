@@ -1,5 +1,5 @@
-// Stage-ring engine of the 512-thread grouped-GEMM kernels, gfx950: mxfp8 tiles and bf16 decode tiles
-// (the wide bf16 tiles use the unit ring of moe_ring128.h, which shares the primitives below).
+// Stage-ring engine of the mxfp8 grouped-GEMM kernels (512 threads), gfx950, and the copy primitives that the
+// bf16 engine (moe_tall.h) shares with it.
 //
 // Tile: token rows x 256 weight rows.  The contraction is consumed in slabs of RB = 64 or 128 bytes
 // per row.  Slabs are copied global -> LDS by the direct-to-LDS path (global_load_lds_*: no staging
@@ -68,7 +68,8 @@ __device__ __forceinline__ Layout make_layout(int ntf0, int ntf1, int budget) {
 // LDS the ring may use, a multiple of 1 KB (the split kernels put their row table behind it).
 template <int DT>
 constexpr int ring_bytes() {
-    return DT == DT_FP8 ? 156 * 1024 : 144 * 1024;
+    static_assert(DT == DT_FP8, "the stage ring serves the mxfp8 kernels");
+    return 156 * 1024;
 }
 
 __device__ __forceinline__ uint32_t lds_addr(const char *p) {
@@ -177,38 +178,6 @@ struct Loader {
     }
 };
 
-struct FragsBf16 {
-    bf16x8 a[2];  // weight fragments
-    bf16x8 b[4];  // token fragments
-};
-
-// Operand fragments of K sub-step j (16 bf16) of a slab: lane l holds row l % 32, chunk 2 j + l / 32.
-template <int RB, int NTF>
-__device__ __forceinline__ void fetch_bf16(FragsBf16 &fr, const char *tok, const char *wgt, const int (&wrow)[2],
-                                           int lane, int j) {
-    const int r = lane & 31, half = lane >> 5, sx = swz<RB>(r);
-    const int off = r * RB + (((2 * j + half) ^ sx) << 4);
-#pragma unroll
-    for (int f = 0; f < 2; ++f) fr.a[f] = *reinterpret_cast<const bf16x8 *>(wgt + wrow[f] * RB + off);
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-        if (t < NTF) fr.b[t] = *reinterpret_cast<const bf16x8 *>(tok + t * 32 * RB + off);
-}
-
-template <int NTF, bool TRANSPOSED>
-__device__ __forceinline__ void mma_bf16(f32x16 (&acc)[2][4], const FragsBf16 &fr) {
-#pragma unroll
-    for (int f = 0; f < 2; ++f)
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-            if (t < NTF) {
-                if constexpr (TRANSPOSED)
-                    acc[f][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.a[f], fr.b[t], acc[f][t], 0, 0, 0);
-                else
-                    acc[f][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.b[t], fr.a[f], acc[f][t], 0, 0, 0);
-            }
-}
-
 // 64 e4m3 of K = one v_mfma_scale_f32_32x32x64_f8f6f4 per (weight fragment, token fragment); `j` is
 // the 64-byte step inside the slab (0 for RB = 64).  Registers 0-3 of both lane halves form K block 0
 // of the step (lanes < 32 its first 16 bytes, lanes >= 32 the last 16), registers 4-7 form K block 1;
@@ -294,17 +263,6 @@ __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader<RB> 
         if (st >= NS) st -= NS;
         if (s < n_slabs) ld.issue(lds + st * SB, rot(s));
     }
-    FragsBf16 fx, fy;  // fy carries the held-back sub-step across the barrier
-    if constexpr (DT == DT_BF16 && COMPUTE) {
-#pragma unroll
-        for (int f = 0; f < 2; ++f)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) fy.a[f][i] = (__bf16)0.0f;
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) fy.b[t][i] = (__bf16)0.0f;
-    }
     const int lps = ld.lps;
     int cur_off = stage0 * SB;  // stage of slab kt
     // stage slab kt + NS - 1 goes to (the one slab kt - 1 used)
@@ -318,21 +276,7 @@ __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader<RB> 
             const char *cur = lds + cur_off;
             const char *tok = cur + tok_region;
             const char *wgt = cur + w_off;
-            if constexpr (DT == DT_BF16) {
-                // software pipeline across the barrier: the last K sub-step of a slab is held back
-                // and issued behind the first fragment reads of the next slab
-                fetch_bf16<RB, NTF>(fx, tok, wgt, wrow, lane, 0);
-                mma_bf16<NTF, TRANSPOSED>(acc, fy);
-#pragma unroll
-                for (int j = 1; j < RB / 32; j += 2) {
-                    fetch_bf16<RB, NTF>(fy, tok, wgt, wrow, lane, j);
-                    mma_bf16<NTF, TRANSPOSED>(acc, fx);
-                    if (j + 1 < RB / 32) {
-                        fetch_bf16<RB, NTF>(fx, tok, wgt, wrow, lane, j + 1);
-                        mma_bf16<NTF, TRANSPOSED>(acc, fy);
-                    }
-                }
-            } else {
+            {
                 const uint32_t *sc = reinterpret_cast<const uint32_t *>(cur + scale_off);
                 const uint32_t *tok_sc = sc + tok_region / RB, *w_sc = sc + scale_tok_rows;
                 if constexpr (RB == 64) {
@@ -351,7 +295,6 @@ __device__ __forceinline__ void main_loop(f32x16 (&acc)[2][4], const Loader<RB> 
         cur_off += SB;
         if (cur_off >= NS * SB) cur_off = 0;
     }
-    if constexpr (DT == DT_BF16 && COMPUTE) mma_bf16<NTF, TRANSPOSED>(acc, fy);
     __syncthreads();  // all reads of the last stages are done: the ring may be reused as scratch
 }
 

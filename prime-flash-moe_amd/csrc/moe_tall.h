@@ -3,9 +3,8 @@
 //
 // Why: a 256 x 256 tile moves 64 KB from L2 to LDS per 2048 matrix-pipe cycles, and that copy path, not
 // the matrix pipe, sets its pace.  A 384 x 256 tile moves 80 KB per 3072 cycles (-17 % bytes per flop).
-// Tiles are cut by 32-row fragments, not by 128-row blocks: an expert with F fragments of rows gets
-// ceil(F / 12) tiles of equal size (+-1 fragment), so no tile streams the expert's weight rows for a
-// handful of rows.
+// Tiles are cut by 32-row fragments, not by 128-row blocks: the tiles of an expert are of equal size (+-1
+// pair of fragments), so no tile streams the expert's weight rows for a handful of rows.
 //
 // A tile has NTF = 2 FG token fragments (FG = 1 .. 6).  Wave (g, v) (g = wave / 4, v = wave % 4) owns
 // token fragments g FG .. g FG + FG - 1 against two 32-row fragments of the weight tile (chosen by the

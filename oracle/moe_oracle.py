@@ -31,6 +31,13 @@ reference checkout) and names the independent checks that pin it
                        Pinned by: dense per-token brute force in fp64, the
                        top_k=1/E=1 reduction to a plain SwiGLU MLP, token
                        permutation equivariance, duplicate-expert additivity.
+  mx_flip_spacing      no counterpart in the reference: which elements of an activation sit so close
+                       to a rounding boundary of its MX quantisation (test/test_mxfp8.py:21-38) that
+                       two evaluations whose fp32 sums differ in order may quantise them to
+                       neighbouring codes, and by how much the dequantised value then differs.
+                       Pinned by: hand-placed values on, next to and away from midpoints and binade
+                       edges; random activations perturbed by less than the margin change only
+                       marked elements, and by no more than the spacing.
   route_topk           the routing the reference's callers do in front of moe_align
                        (README.md:147-149): top-k of the gate logits by value,
                        largest first, ties to the lower expert index, softmax over
@@ -299,8 +306,40 @@ def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return up * gate / (1.0 + torch.exp(-gate))
 
 
+def mx_flip_spacing(act: torch.Tensor, delta: float, block: int = BLOCK) -> torch.Tensor:
+    """Per element of ``act`` (rows x H, H % 32 == 0): 0 if the MX quantisation of the element
+    (test/test_mxfp8.py:21-38: shared power-of-two scale per 32 elements from the block's amax, e4m3 values,
+    round to nearest even, saturating) cannot change when every element moves by less than the relative
+    distance ``delta``; otherwise the largest change of its dequantised value, which is the spacing of the
+    e4m3 grid at that value times the block's scale:
+      * the scaled value lies within ``delta`` (relative) of the midpoint of two neighbouring codes: one
+        spacing;
+      * the block's amax lies within ``delta`` of a power of two, so that the shared scale may come out one
+        step larger or smaller: every element of the block, one spacing of the coarser of the two grids.
+    Math in float64."""
+    n, H = act.shape
+    a = act.double().abs().view(n, H // block, block)
+    amax = a.amax(-1)
+    # the quantiser's scale: 2^(expfield(amax as fp32) - 8 - 127), expfield clamped as in shared_exponent
+    bits = amax.float().view(torch.int32).to(torch.int64)
+    e = (((bits >> 23) & 0xff) - E4M3_EMAX).clamp(0, 254)
+    scale = torch.pow(torch.tensor(2.0, dtype=torch.float64, device=act.device), (e - 127).double()).unsqueeze(-1)
+    s = a / scale
+    # spacing of the e4m3 grid at |s|: 2^(floor(log2 s) - 3), binades from 2^-6 (below: subnormals, 2^-9) to 2^8
+    _, ex = torch.frexp(s.clamp_min(2.0 ** -20))
+    ex = (ex - 1).clamp(-6, 8)
+    ulp = torch.pow(torch.tensor(2.0, dtype=torch.float64, device=act.device), (ex - 3).double())
+    q = s / ulp
+    near_mid = ((q - torch.floor(q) - 0.5).abs() <= delta * q) & (s < E4M3_MAX + 16.0)  # (beyond 464 everything saturates)
+    m, _ = torch.frexp(amax.clamp_min(2.0 ** -140))  # amax = m * 2^k, m in [0.5, 1)
+    near_pow2 = (((m - 0.5) <= delta * 0.5) | ((1.0 - m) <= delta)) & (amax > 0)
+    spacing = torch.where(near_mid, ulp, torch.zeros_like(ulp))
+    spacing = torch.where(near_pow2.unsqueeze(-1), 2.0 * ulp, spacing)
+    return (spacing * scale).view(n, H)
+
+
 def fused_moe_dense(x, w1, w2, topk_ids, topk_weights, act_mx: bool = False,
-                    dtype=torch.float32) -> torch.Tensor:
+                    dtype=torch.float32, flip_delta: float = None):
     """out[t] = sum_r w[t,r] * W2[e] @ swiglu(W1[e] @ x[t]),  e = topk_ids[t,r].
 
     Dataflow of test/test.py:13-48 (grouped by expert), all math in ``dtype``
@@ -309,12 +348,17 @@ def fused_moe_dense(x, w1, w2, topk_ids, topk_weights, act_mx: bool = False,
     the down projection (test_mxfp8.py:70-72; kernel: fused_moe_mxfp8_kernel.cu:375-403,
     which requantises the fp32 SwiGLU value directly).
     x:(T,K) w1:(E,2H,K) w2:(E,K,H) topk_ids:(T,k) int, topk_weights:(T,k).
+    ``flip_delta`` (with act_mx): also returns, per output element, how far another evaluation of the same
+    dataflow may lie from this one because activations within that relative distance of a rounding boundary
+    were quantised to the neighbouring code (see mx_flip_spacing): sum over the token's pairs of
+    w * spacing . |W2[e]|; the activations that decide this are computed in float64.
     """
     T, K = x.shape
     E, N, _ = w1.shape
     H = N // 2
     xf = x.to(dtype)
     out = torch.zeros((T, K), dtype=dtype)
+    bound = torch.zeros((T, K), dtype=torch.float64) if flip_delta is not None else None
     ids = topk_ids.to(torch.int64)
     wts = topk_weights.to(dtype)
     for e in range(E):
@@ -324,24 +368,31 @@ def fused_moe_dense(x, w1, w2, topk_ids, topk_weights, act_mx: bool = False,
         h = xf[tok] @ w1[e].to(dtype).t()
         act = swiglu(h[:, :H], h[:, H:])
         if act_mx:
+            if bound is not None:
+                h64 = x[tok].double() @ w1[e].double().t()
+                sp = mx_flip_spacing(swiglu(h64[:, :H], h64[:, H:]), flip_delta)
+                bound.index_add_(0, tok, (sp @ w2[e].double().abs().t()) * wts[tok, slot].double().abs()[:, None])
             q, s = quantize_mx_torch(act.float())
             act = dequantize_mx_torch(q, s).to(dtype)
         y = act @ w2[e].to(dtype).t()
         out.index_add_(0, tok, y * wts[tok, slot][:, None])
-    return out
+    return out if bound is None else (out, bound)
 
 
 def fused_moe_by_expert(x, expert_weights, topk_ids, topk_weights, num_experts: int, act_mx: bool = False,
-                        experts=None, dtype=torch.float32) -> torch.Tensor:
+                        experts=None, dtype=torch.float32, flip_delta: float = None):
     """fused_moe_dense with the weights fetched one expert at a time: ``expert_weights(e)`` returns
     ``(w1_e (2H, K), w2_e (K, H))`` (already dequantised for mxfp8) on the device of ``x``.  Keeps the
     memory of a full-size configuration bounded, and runs wherever ``x`` lives.  ``experts``: only
     these experts contribute (the pairs routed elsewhere add nothing), for checks on a subset.
     Same dataflow and citations as fused_moe_dense; pinned against it in tests/test_oracle.py.
+    ``flip_delta``: as in fused_moe_dense, except that the activations that decide the bound are the ``dtype``
+    ones (a full-size configuration in float64 would take too long): choose a margin that covers their error.
     """
     T, K = x.shape
     xf = x.to(dtype)
     out = torch.zeros((T, K), dtype=dtype, device=x.device)
+    bound = torch.zeros((T, K), dtype=torch.float64, device=x.device) if flip_delta is not None else None
     ids = topk_ids.to(torch.int64)
     wts = topk_weights.to(dtype)
     todo = range(num_experts) if experts is None else sorted(int(e) for e in experts)
@@ -354,11 +405,14 @@ def fused_moe_by_expert(x, expert_weights, topk_ids, topk_weights, num_experts: 
         h = xf[tok] @ w1.to(dtype).t()
         act = swiglu(h[:, :H], h[:, H:])
         if act_mx:
+            if bound is not None:
+                sp = mx_flip_spacing(act, flip_delta)
+                bound.index_add_(0, tok, (sp @ w2.double().abs().t()) * wts[tok, slot].double().abs()[:, None])
             q, s = quantize_mx_torch(act.float())
             act = dequantize_mx_torch(q, s).to(dtype)
         y = act @ w2.to(dtype).t()
         out.index_add_(0, tok, y * wts[tok, slot][:, None])
-    return out
+    return out if bound is None else (out, bound)
 
 
 def fused_moe_sorted(x, w1, w2, sorted_token_ids, expert_ids, num_tokens_post_padded,

@@ -11,11 +11,32 @@ MX_RELL2_GATE = 2e-2    # ||got - ref|| / ||ref|| ceiling for the mxfp8 path
 # :168-191): max |got - ref| / max(|ref|, c) for c = 1 and c = 10
 MX_REL_CLAMP_1_GATE = 2e-2
 MX_REL_CLAMP_10_GATE = 2e-3
+# An activation within this relative distance of a rounding boundary of its MX quantisation may come out on the
+# neighbouring code in two evaluations that add the same fp32 products in different orders (kernel and oracle);
+# the oracle bounds what that does to every output element (oracle.mx_flip_spacing), and the element-wise gates
+# allow that much on top of the reference's thresholds, and nothing else.
+MX_FLIP_DELTA = 1e-4
 
 
 def rel_clamp(got: torch.Tensor, ref: torch.Tensor, c: float) -> float:
     d = (got.double() - ref.double()).abs()
     return float((d / ref.double().abs().clamp_min(c)).max())
+
+
+def mx_elementwise_gates(got: torch.Tensor, ref: torch.Tensor, bound: torch.Tensor):
+    """The reference's element-wise gates (test/test_mxfp8.py:168-191) on what is left of |got - ref| after the
+    oracle's bound on boundary flips of the activation quantisation (MX_FLIP_DELTA) is taken off: elements that no
+    such flip can reach (bound 0: most of them) face the reference's thresholds exactly.  Returns
+    (rel_clamp_1, rel_clamp_10, elements that needed the bound)."""
+    d = (got.double() - ref.double()).abs()
+    rest = (d - bound.double().to(d.device)).clamp_min(0.0)
+    a = ref.double().abs()
+    rc1 = float((rest / a.clamp_min(1.0)).max())
+    rc10 = float((rest / a.clamp_min(10.0)).max())
+    needed = int(((d > MX_REL_CLAMP_1_GATE * a.clamp_min(1.0)) | (d > MX_REL_CLAMP_10_GATE * a.clamp_min(10.0))).sum())
+    assert rc1 <= MX_REL_CLAMP_1_GATE, f"rel_clamp_1 {rc1} beyond what boundary flips explain ({needed} elements over the plain gates)"
+    assert rc10 <= MX_REL_CLAMP_10_GATE, f"rel_clamp_10 {rc10} beyond what boundary flips explain ({needed} elements over the plain gates)"
+    return rc1, rc10, needed
 
 
 def cosine(got: torch.Tensor, ref: torch.Tensor) -> float:

@@ -351,3 +351,53 @@ def test_forward_by_expert_equals_dense_and_subset_masks():
         masked = O.fused_moe_dense(x, w1, w2, ids, wts * keep, act_mx=act_mx)
         torch.testing.assert_close(O.fused_moe_by_expert(x, fetch, ids, wts, 5, act_mx=act_mx, experts=[3, 1]),
                                    masked, rtol=1e-6, atol=1e-6)
+
+
+def test_mx_flip_spacing_marks_what_can_flip_and_bounds_the_change():
+    # hand-placed values in one block whose amax 3.0 gives the scale 2^-7 (scaled amax 384, spacing 32 there):
+    # 0.40625 = 52 * 2^-7 is a code (spacing 4 in [32, 64)), 0.421875 = 54 * 2^-7 the midpoint to the next one
+    # (56), 0.4296875 = 55 * 2^-7 lies a quarter spacing from it
+    row = torch.zeros(32, dtype=torch.float64)
+    row[0], row[1], row[2], row[3] = 3.0, 0.40625, 0.421875, 0.4296875
+    row[4] = 0.421875 * (1 + 5e-5)   # within 1e-4 of the midpoint
+    row[5] = 0.421875 * (1 + 3e-4)   # outside
+    sp = O.mx_flip_spacing(row.view(1, 32), 1e-4)[0]
+    assert sp[0] == 0 and sp[1] == 0 and sp[3] == 0 and sp[5] == 0
+    assert sp[2] == 4 * 2.0 ** -7 and sp[4] == 4 * 2.0 ** -7
+    # amax next to a power of two: the scale may come out either way, the whole block is marked with the spacing
+    # of the coarser grid
+    row2 = row.clone()
+    row2[0] = 4.0 * (1 - 2e-5)
+    sp2 = O.mx_flip_spacing(row2.view(1, 32), 1e-4)[0]
+    assert (sp2 > 0).all() and sp2[1] == 2 * 4 * 2.0 ** -7
+    # random activations moved by less than the margin: only marked elements change, by no more than the spacing
+    g = torch.Generator().manual_seed(4)
+    act = torch.randn((128, 256), generator=g, dtype=torch.float64) * 3
+    sp = O.mx_flip_spacing(act, 1e-4)
+    assert 0 < float((sp > 0).double().mean()) < 0.01
+    changed = 0
+    for _ in range(8):
+        moved = act * (1 + (torch.rand(act.shape, generator=g, dtype=torch.float64) * 2 - 1) * 0.9e-4)
+        d0 = O.dequantize_mx_torch(*O.quantize_mx_torch(act.float())).double()
+        d1 = O.dequantize_mx_torch(*O.quantize_mx_torch(moved.float())).double()
+        diff = (d0 - d1).abs()
+        assert bool((diff <= sp + 1e-12).all())
+        changed += int((diff > 0).sum())
+    assert changed > 0
+
+
+def test_flip_bound_of_the_forward_pass():
+    # the bound is zero where no activation can flip, and covers the difference between two evaluations of the
+    # forward pass whose activations differ by less than the margin
+    g = torch.Generator().manual_seed(9)
+    T, K, E, N, top_k = 24, 64, 3, 128, 2
+    x = torch.randn((T, K), generator=g)
+    w1 = torch.randn((E, N, K), generator=g) / K ** 0.5
+    w2 = torch.randn((E, K, N // 2), generator=g) / (N // 2) ** 0.5
+    ids = torch.stack([torch.randperm(E, generator=g)[:top_k] for _ in range(T)]).to(torch.int32)
+    wts = torch.softmax(torch.randn((T, top_k), generator=g), -1)
+    ref, bound = O.fused_moe_dense(x, w1, w2, ids, wts, act_mx=True, flip_delta=1e-4)
+    assert bound.shape == ref.shape and float(bound.min()) >= 0
+    other = O.fused_moe_dense(x * (1 + 2e-5), w1, w2, ids, wts, act_mx=True)  # every activation moves by ~4e-5
+    rest = ((other.double() - ref.double()).abs() - bound).clamp_min(0)
+    assert float(rest.max()) <= 2e-4 * float(ref.abs().max())

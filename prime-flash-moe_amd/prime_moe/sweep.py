@@ -16,7 +16,9 @@ tokens 4096 ... 131072, both dtypes, split=True, median of per-iteration event t
 reference's, the run can be shaped from the command line (``bench.py --sweep``): experts, top_k, hidden and
 intermediate size, ``balancedness`` of the routing (benchmark.py:116-121: every (token, slot) draws its
 expert from ``b * uniform + (1 - b) * all-to-expert-0``, with replacement), seed, and whether the timed
-callables are graph replays (benchmark.py:355-370, the reference's default) or eager calls.
+callables are graph replays (benchmark.py:355-370, the reference's default) or eager calls.  A row never mixes
+the two: if one of its callables cannot be captured (or its replay does not reproduce the eager result), every
+callable of the row is timed eagerly, and the columns ``timed_as`` / ``timed_note`` say so and why.
 """
 from __future__ import annotations
 
@@ -24,6 +26,7 @@ import csv
 import math
 import statistics
 import sys
+import warnings
 
 import torch
 import torch.nn.functional as F
@@ -32,7 +35,7 @@ import prime_moe
 
 COLUMNS = ["dtype", "tokens", "E", "K", "N", "top_k", "naive_ms", "baseline_ms", "noreq_ms", "fused_ms", "speedup",
            "speedup_noreq", "speedup_naive", "naive_tflops", "baseline_tflops", "fused_tflops", "max_abs", "rel",
-           "naive_max_abs", "baseline_kind", "split"]
+           "naive_max_abs", "baseline_kind", "split", "timed_as", "timed_note"]
 
 
 def median_ms(fn, warmup: int, iters: int) -> float:
@@ -50,24 +53,32 @@ def median_ms(fn, warmup: int, iters: int) -> float:
     return statistics.median(times)
 
 
-def graphed(fn, warmup: int = 3):
-    """`fn` captured into a graph after a warm-up on a side stream; None if the capture fails (the
-    reference's recipe, benchmark.py:355-370: the caller then times `fn` eagerly)."""
+def capture_replay(fn, reproduces=None):
+    """Records one call of `fn` in a HIP graph.  Returns (replay, None), or (None, reason) when the call cannot
+    be recorded: it raises under capture (a host synchronisation, an allocation the capture forbids), it records
+    nothing (torch warns of an empty graph: the work went to another stream), or `reproduces(replay)`, the
+    caller's check that a replay gives what an eager call gives, says no."""
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    reason = None
     try:
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for _ in range(warmup):
-                fn()
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
+        with torch.cuda.stream(stream):  # first calls outside the capture: lazy initialisation, allocator warm-up
             fn()
-        return g.replay
-    except Exception:
+            fn()
+        torch.cuda.current_stream().wait_stream(stream)
         torch.cuda.synchronize()
-        return None
+        with warnings.catch_warnings():
+            warnings.simplefilter("error")  # "The CUDA Graph is empty" must not pass for a recording
+            with torch.cuda.graph(graph):
+                fn()
+    except (RuntimeError, Warning) as exc:
+        text = str(exc).strip()
+        reason = f"{type(exc).__name__}: {text.splitlines()[0] if text else 'no message'}"
+    torch.cuda.synchronize()
+    if reason is None and reproduces is not None and not reproduces(graph.replay):
+        reason = "a replay does not reproduce the eager result"
+    return (graph.replay, None) if reason is None else (None, reason)
 
 
 def generate_topk_ids(E: int, tokens: int, top_k: int, balancedness: float, gen: torch.Generator) -> torch.Tensor:
@@ -168,12 +179,30 @@ def run_one(dtype: str, tokens: int, E: int, K: int, H: int, top_k: int, split: 
         diff = (ref.float() - got).abs()
         max_abs, rel = float(diff.max()), float((diff / ref.float().abs().clamp_min(1.0)).max())
     timed = {"baseline": baseline, "naive": naive, "fused": step}
+    timed_as, timed_note = "eager", ""
     if graphs:
+        def fused_reproduces(replay):
+            # one replay must rewrite a poisoned `out` to the bits of an eager call
+            step()
+            torch.cuda.synchronize()
+            want = out.clone()
+            out.fill_(float("nan"))
+            replay()
+            torch.cuda.synchronize()
+            return bool(torch.equal(out.view(torch.int16), want.view(torch.int16)))
+
+        replays, why = {}, []
         for name in ("baseline", "fused") + (() if skip_naive else ("naive",)):
-            replay = graphed(timed[name])
-            if replay is None and log is not None:
-                log(f"  note: graph capture failed for the {name} callable, timing it eagerly")
-            timed[name] = replay or timed[name]
+            replays[name], reason = capture_replay(timed[name], fused_reproduces if name == "fused" else None)
+            if reason is not None:
+                why.append(f"{name}: {reason}")
+        if why:  # never a replayed callable next to an eager one
+            timed_note = "graph replays asked for, all callables timed eagerly; " + "; ".join(why)
+            if log is not None:
+                log("  note: " + timed_note)
+        else:
+            timed.update(replays)
+            timed_as = "replay"
     baseline_ms = median_ms(timed["baseline"], warmup, iters)
     naive_ms = float("nan") if skip_naive else median_ms(timed["naive"], warmup, iters)
     fused_ms = median_ms(timed["fused"], warmup, iters)
@@ -183,7 +212,8 @@ def run_one(dtype: str, tokens: int, E: int, K: int, H: int, top_k: int, split: 
             "baseline_ms": baseline_ms, "noreq_ms": float("nan"), "fused_ms": fused_ms, "speedup": baseline_ms / fused_ms,
             "speedup_noreq": float("nan"), "speedup_naive": naive_ms / fused_ms, "naive_tflops": tf(naive_ms),
             "baseline_tflops": tf(baseline_ms), "fused_tflops": tf(fused_ms), "max_abs": max_abs, "rel": rel,
-            "naive_max_abs": naive_max_abs, "baseline_kind": kind, "split": int(split)}
+            "naive_max_abs": naive_max_abs, "baseline_kind": kind, "split": int(split), "timed_as": timed_as,
+            "timed_note": timed_note}
 
 
 def run_sweep(path: str, tokens=(4096, 8192, 16384, 32768, 65536, 131072), dtypes=("bf16", "mxfp8"), E=32, top_k=4,
@@ -198,7 +228,7 @@ def run_sweep(path: str, tokens=(4096, 8192, 16384, 32768, 65536, 131072), dtype
             log(f"{dtype:6s} tokens {t:7d}: fused {r['fused_ms']:8.3f} ms ({r['fused_tflops']:7.1f} TFLOP/s)  "
                 f"{r['baseline_kind']} {r['baseline_ms']:8.3f} ms  speedup {r['speedup']:.2f}x  "
                 f"naive loop {r['naive_ms']:8.3f} ms  max_abs {r['max_abs']:.3g} rel {r['rel']:.3g}"
-                + ("  (graph replays)" if graphs else ""))
+                + f"  ({r['timed_as']})")
             torch.cuda.empty_cache()
     with open(path, "w", newline="") as f:
         w = csv.DictWriter(f, fieldnames=COLUMNS)

@@ -43,6 +43,14 @@ void pmoe_set_tiles_per_workgroup(int n);
  */
 int pmoe_copy_calibration(const void *src, void *dst, int64_t bytes, void *stream);
 
+/*
+ * Test aid without a counterpart in the reference: fills the LDS of every CU with 0xff bytes (NaN as bf16, e4m3
+ * and e8m0), so that a kernel launched next which reads LDS that its own copies did not fill (a direct-to-LDS copy
+ * that landed in the wrong place) produces NaNs instead of whatever an earlier kernel left behind.
+ * `scratch_word`: one int of device memory (written only if the fill itself misbehaves).
+ */
+int pmoe_poison_lds(int *scratch_word, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -75,9 +75,15 @@ constexpr int ring_bytes() {
 __device__ __forceinline__ uint32_t lds_addr(const char *p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
 }
-// (M0 is written inside the statements without being declared: the compiler reserves the register and
-// rejects it in a clobber list.  Nothing in these kernels makes the compiler itself keep a value in M0
-// across a statement: no LDS-DMA builtin, no register-indexed moves, accumulators indexed by constants.)
+// M0 holds the LDS address of a direct-to-LDS copy.  The statements below write it without declaring it: the
+// compiler reserves the register and rejects it in a clobber list.  That is sound only while the compiler itself
+// keeps no value in M0 across a statement, so the kernels that use these primitives stay clear of everything that
+// makes it use M0 on gfx950: the LDS-DMA builtins (__builtin_amdgcn_global_load_lds, raw_buffer_load_lds), GWS
+// and s_sendmsg builtins, register-indexed moves (accumulators and fragment arrays are indexed by constants after
+// unrolling only), readlane / writelane with a lane number that is not a compile-time constant.  A host test
+// compiles the two translation units that include this file to assembly and fails if a kernel that contains a
+// copy touches M0 anywhere outside these statements (tests/test_host.py); a GPU test runs the tile paths with the
+// most copies between two barriers on poisoned LDS (tests/test_gpu_lds_copies.py).
 __device__ __forceinline__ void copy16(const char *base, uint32_t voff, const char *lds_dst) {
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base), "s"(lds_addr(lds_dst)) : "memory");
 }

@@ -32,6 +32,7 @@ SIGNATURES = {
     "pmoe_set_phase_mask": (None, [_c_int]),
     "pmoe_set_tiles_per_workgroup": (None, [_c_int]),
     "pmoe_copy_calibration": (_c_int, [_c_void_p, _c_void_p, ctypes.c_int64, _c_void_p]),
+    "pmoe_poison_lds": (_c_int, [_c_void_p, _c_void_p]),
 }
 
 _lib = None

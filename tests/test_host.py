@@ -33,7 +33,8 @@ def test_library_exports_every_declared_symbol():
 def test_workspace_query_and_c_side_validation_need_no_gpu():
     from prime_moe import _native
     lib = _native.load()
-    # bf16: plan (256 B) + run list and the two tables of row tiles (16 B per block + 1 each) + fp32 partial sums of
+    # bf16: plan (256 B) + run list with its order (20 B per block + 1) + the two tables of row tiles (16 B per block
+    # + 1 each) + fp32 partial sums of
     # the deep contraction split when the problem has at most 32 (block, up weight tile) pairs and K >= 2048
     # (8 parts x 32 KB per fragment and weight tile) + inverse of the sorted order (4 B per pair) + y (one row of
     # K bf16 per pair) + act (rows * H bf16), each rounded to 256 B; the same for both values of split
@@ -43,7 +44,7 @@ def test_workspace_query_and_c_side_validation_need_no_gpu():
         lib.pmoe_fused_moe_bf16_workspace_bytes(256, 4096, 512, 8, 2048, 4, 1)
     # no partial sums are reserved for a problem too large for the deep split
     assert lib.pmoe_fused_moe_bf16_workspace_bytes(4096, 4096, 28672, 8, 9216, 2, 1) == \
-        256 + 3 * 1280 + 8192 * 4 + 8192 * 4096 * 2 + 9216 * 14336 * 2
+        256 + 1536 + 2 * 1280 + 8192 * 4 + 8192 * 4096 * 2 + 9216 * 14336 * 2
     # mxfp8: header (256 B) + row-tile list (8 B per block) + the two work lists (16 B per block and weight tile)
     # + inverse of the sorted order + y + act (rows * H e4m3) + act scales + re-tiled x scales
     assert lib.pmoe_fused_moe_mxfp8_workspace_bytes(64, 7168, 4096, 256, 33024, 8, 1) == \
@@ -243,3 +244,48 @@ def test_sweep_routing_and_columns_on_the_host():
     assert sweep.COLUMNS[6:19] == ["naive_ms", "baseline_ms", "noreq_ms", "fused_ms", "speedup", "speedup_noreq",
                                    "speedup_naive", "naive_tflops", "baseline_tflops", "fused_tflops", "max_abs", "rel",
                                    "naive_max_abs"]
+
+
+def test_no_compiler_use_of_m0_in_kernels_with_direct_to_lds_copies(tmp_path):
+    """The copy primitives of csrc/moe_ring.h set M0 inside inline assembly without telling the compiler.  Enforced
+    here: in the device assembly of every translation unit that includes them, a kernel that contains such a copy
+    names M0 only between the markers of those statements, and the sources use none of the builtins that would
+    make the compiler hold a value in M0."""
+    import glob
+    import re
+    import subprocess
+    from prime_moe import build
+    csrc = build.CSRC
+    users = [f for f in glob.glob(os.path.join(csrc, "*.hip")) if "moe_ring.h" in open(f).read() or "moe_tall.h" in open(f).read()]
+    assert len(users) == 2, users
+    banned = re.compile(r"__builtin_amdgcn_(global_load_lds|raw_buffer_load_lds|struct_buffer_load_lds|ds_gws\w*|s_sendmsg\w*|"
+                        r"s_movrel\w*|mov_dpp8)")
+    for f in users + [os.path.join(csrc, h) for h in ("moe_ring.h", "moe_tall.h", "moe_tile.h", "moe_pipeline.h")]:
+        text = re.sub(r"//[^\n]*", "", open(f).read())  # (the header's comment names them)
+        assert not banned.search(text), (f, banned.search(text).group(0))
+    for f in users:
+        asm = tmp_path / (os.path.basename(f) + ".s")
+        cmd = [build.hipcc(), f"--offload-arch={build.ARCH}", "-O3", "-std=c++17", "-munsafe-fp-atomics", *build.DEVICE_FLAGS,
+               "-S", "--cuda-device-only", f, "-o", str(asm)]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        assert res.returncode == 0, res.stderr[-2000:]
+        kernel, in_asm, copies, stray = None, False, {}, {}
+        for line in open(asm):
+            m = re.match(r"^(_Z\w+):", line)
+            if m:
+                kernel = m.group(1)
+            if ";;#ASMSTART" in line:
+                in_asm = True
+            elif ";;#ASMEND" in line:
+                in_asm = False
+            code = line.split(";")[0]
+            if kernel is None or not code.strip() or code.lstrip().startswith("."):
+                continue
+            if "global_load_lds" in code:
+                assert in_asm, (kernel, line)  # only the hand-issued ones exist
+                copies[kernel] = copies.get(kernel, 0) + 1
+            if re.search(r"\bm0\b", code) and not in_asm:
+                stray.setdefault(kernel, []).append(line.strip())
+        assert copies, f"{f}: no direct-to-LDS copy found in the assembly"
+        for k in copies:
+            assert k not in stray, (k, stray[k][:5])

@@ -69,7 +69,7 @@ int pmoe_moe_align_ws(const int32_t *topk_ids, int32_t *sorted_token_ids, int32_
  * The same sort for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc); no counterpart in the reference.
  * Takes what pmoe_moe_align takes and gives the same output, bit for bit, but the scratch of
- * the multi-workgroup sort lives in a device array built into the library (516 KB on every
+ * the multi-workgroup sort lives in a device array built into the library (520 KB on every
  * device the library runs on, held until the process ends), so large inputs still spread
  * over many workgroups.  n > PMOE_ALIGN_STATIC_MAX_IDS is rejected (PMOE_ERR_INVALID).
  * Calls no hipMalloc / hipFree or any allocating routine; the first call on a device looks
@@ -110,6 +110,9 @@ size_t pmoe_fused_moe_mxfp8_workspace_bytes(int M, int K, int N, int num_experts
  * num_experts <= 1024 (as moe_align) and x smaller than 4 GiB.
  * The workspace is scratch of this one call: calls that may run at the same time need
  * their own.
+ * A schedule that lists a pair id twice: inside one block the pair contributes once; in blocks
+ * of different experts one of the two rows stands for the pair, which one is unspecified
+ * (nothing faults, the rest of the output is unaffected).
  */
 int pmoe_fused_moe_bf16(const void *x, const void *w, const void *w2, void *out,
                         const int32_t *sorted_token_ids, const int32_t *expert_idxs,

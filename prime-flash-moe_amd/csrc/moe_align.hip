@@ -295,7 +295,7 @@ __global__ __launch_bounds__(NW * 64) void align_scatter_kernel(const int32_t *_
 
 
 // Scratch of the entry point that allocates nothing (pmoe_moe_align_static): counts[G][E], offs[E + 1],
-// cnt[E] of the multi-workgroup sort for up to kStaticMaxIds ids and kMaxExperts experts, 516 KB held by
+// cnt[E] of the multi-workgroup sort for up to kStaticMaxIds ids and kMaxExperts experts, 520 KB held by
 // every device the library runs on until the process ends.  In host code this name is only a handle for
 // hipGetSymbolAddress; kernels get the address that call returns.
 constexpr int kStaticMaxIds = PMOE_ALIGN_STATIC_MAX_IDS;
@@ -374,16 +374,23 @@ int launch_multi(const int32_t *topk_ids, int32_t *sorted_token_ids, int32_t *ex
 }
 
 // Device address of `scratch` on the current device: every device holds its own copy of the array at
-// its own address, looked up once per device (with that device current) and kept.
+// its own address, looked up once per device (with that device current) and kept.  `data` is one of the
+// call's device pointers: the current device must be the one that holds it (the kernels run where the data
+// is, and another device's copy of the array has another address), otherwise the call is rejected.
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 int32_t *g_scratch_ptr[kMaxDevices] = {nullptr};
 
-int static_scratch(int32_t **out) {
+int static_scratch(const void *data, int32_t **out) {
     int dev = 0;
     hipError_t err = hipGetDevice(&dev);
     if (err != hipSuccess) return pmoe::fail(PMOE_ERR_HIP, "moe_align_static: hipGetDevice: %s", hipGetErrorString(err));
     PMOE_REQUIRE(dev >= 0 && dev < kMaxDevices, "moe_align_static: device index %d out of range", dev);
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, data) == hipSuccess)
+        PMOE_REQUIRE(attr.device == dev, "moe_align_static: the data lives on device %d but device %d is current", attr.device, dev);
+    else
+        (void)hipGetLastError();  // (a pointer the runtime does not know: nothing to compare)
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (g_scratch_ptr[dev] == nullptr) {
         void *p = nullptr;
@@ -442,7 +449,7 @@ extern "C" int pmoe_moe_align_static(const int32_t *topk_ids, int32_t *sorted_to
         return launch_single(topk_ids, sorted_token_ids, expert_ids, num_tokens_post_padded, n, num_experts, block_m,
                              pad_to, max_padded, max_blocks, s);
     int32_t *words = nullptr;
-    if (int rc = static_scratch(&words)) return rc;
+    if (int rc = static_scratch(topk_ids, &words)) return rc;
     return launch_multi(topk_ids, sorted_token_ids, expert_ids, num_tokens_post_padded, n, num_experts, block_m,
                         pad_to, max_padded, max_blocks, words, s);
 }

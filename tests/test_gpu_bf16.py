@@ -185,8 +185,9 @@ def test_experts_with_one_and_with_several_row_tiles(device):
 
 def test_block_without_expert_and_duplicate_pair(device):
     """Schedules the fused op must survive: a block whose expert id is out of range is not computed and
-    its pairs contribute nothing (never whatever the workspace held); a pair id listed twice contributes
-    once."""
+    its pairs contribute nothing (never whatever the workspace held); a pair id listed twice in one block
+    contributes once; listed again in a block of another expert, one of the two experts' rows (unspecified
+    which) stands for the pair, and nothing faults."""
     import prime_moe
     T, K, E, N, top_k = 300, 512, 6, 512, 2
     g, x, w1, w2 = _inputs(T, K, E, N, device, seed=9)
@@ -219,6 +220,24 @@ def test_block_without_expert_and_duplicate_pair(device):
         prime_moe.fused_moe_bf16(x, w1, w2, s_dup, e, n, wts, out, top_k, 128, 64, 4, 2, 1, 1, True)
         torch.cuda.synchronize()
         assert rel_clamp(out.float().cpu(), ref, 1.0) <= BF16_GATE
+    # the same pair id once more in a padding slot of another expert's block: two workgroups write y[pair]; the
+    # result for that token is one of the two candidates, the rest of the output is untouched
+    other = [b for b in range(1, int(n[0]) // 128) if int(e[b]) != int(e[0]) and bool((s[b * 128:(b + 1) * 128] < 0).any())]
+    if other:
+        b = other[0]
+        slot = b * 128 + int((s[b * 128:(b + 1) * 128] < 0).nonzero()[0])
+        s_far = s.clone()
+        s_far[slot] = s[0]
+        ref = O.fused_moe_dense(x.cpu(), w1.cpu(), w2.cpu(), ids.cpu(), wts.cpu())
+        out = torch.empty((T, K), dtype=torch.bfloat16, device=device)
+        prime_moe.fused_moe_bf16(x, w1, w2, s_far, e, n, wts, out, top_k, 128, 64, 4, 2, 1, 1, True)
+        torch.cuda.synchronize()
+        got = out.float().cpu()
+        assert torch.isfinite(got).all()
+        tok = int(s[0]) // top_k
+        keep = torch.ones(T, dtype=torch.bool)
+        keep[tok] = False
+        assert rel_clamp(got[keep], ref[keep], 1.0) <= BF16_GATE
 
 
 @pytest.mark.parametrize("T,K,E,N,top_k,exact", [

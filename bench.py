@@ -379,6 +379,10 @@ def main():
                     continue
                 everything.append(summary(run_config(cfg, split, args.steps, args.warmup, device, False, log)))
                 torch.cuda.empty_cache()
+        from prime_moe.workloads import GRID_CONFIGS
+        for cfg in GRID_CONFIGS.values():
+            everything.append(summary(run_config(cfg, 1, args.steps, args.warmup, device, False, log)))
+            torch.cuda.empty_cache()
         router = router_times(device, 20)
         log(f"router front-end on {router['workload']}: fused {router['fused_us']:.1f} us, "
             f"torch top-k + softmax + moe_align op {router['unfused_us']:.1f} us")

@@ -52,6 +52,13 @@ CONFIGS: Dict[str, MoeConfig] = {
     "c5_decode_mxfp8": MoeConfig("c5_decode_mxfp8", "mxfp8", 64, 7168, 256, 4096, 8, "zipf"),
 }
 
+# The compute-bound end of the reference benchmark's own grid (benchmark/benchmark.py:695-718: E=32, top_k=4,
+# K=2048, H=1024, 131072 tokens, 16384 rows per expert): reported next to the five specification workloads.
+GRID_CONFIGS: Dict[str, MoeConfig] = {
+    "g1_grid_bf16_131072": MoeConfig("g1_grid_bf16_131072", "bf16", 131072, 2048, 32, 2048, 4, "topk"),
+    "g2_grid_mxfp8_131072": MoeConfig("g2_grid_mxfp8_131072", "mxfp8", 131072, 2048, 32, 2048, 4, "topk"),
+}
+
 
 def make_routing(cfg: MoeConfig, gen: torch.Generator, device) -> Dict[str, torch.Tensor]:
     """topk_ids (T, top_k) int32 and topk_weights (T, top_k) fp32 for the config's routing rule."""

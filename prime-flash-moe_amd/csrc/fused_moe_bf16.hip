@@ -33,8 +33,9 @@ __device__ __forceinline__ int block_scan(int v, int *s_part) {
 
 // Estimated time of a kernel (in units of a third of a microsecond) whose `f2` pairs of fragments are cut into
 // `n_tiles` row tiles: whole rounds of the chip's CUs at the cost of a mean tile, plus a last round whose jobs
-// are shared by rows.  A tile of g pairs costs (0.6 + g) per slab of its K loop (measured: 0.18 + 0.34 g us on
-// tiles of 2 to 6 pairs) and 3 + 2.5 g for set-up and epilogue; a round of nothing but shared jobs costs 1.3
+// are shared by rows.  A tile of g pairs costs (0.6 + g) per slab of its K loop (measured on operands that stay in
+// L2: 0.18 + 0.34 g us on tiles of 2 to 6 pairs; inside a full kernel the fixed part is larger, which only
+// strengthens the preference for few, tall tiles) and 3 + 2.5 g for set-up and epilogue; a round of nothing but shared jobs costs 1.3
 // times what its small tiles would among large ones (measured on the Mixtral-like down kernel: every weight row
 // is then read twice as often).
 __device__ __forceinline__ float estimate_kernel(int n_tiles, int f2, int n_wt, int n_slabs, int n_cus, int &parts,

@@ -399,13 +399,13 @@ def main():
         n_touched = int(torch.unique(r["topk_ids"]).numel())
         up_bytes = (n_touched * cfg.N * cfg.K + P * cfg.K + P * cfg.H) * 33 // 32
         roofline = {"bound": "hbm", "achieved": up_bytes / r["t_up"] / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "kernel": "moe_up_kernel (gate/up GEMM + SwiGLU + requantisation)",
+                    "kernel": "moe_up_kernel<1> (mxfp8 gate/up GEMM + SwiGLU + requantisation)",
                     "launch_us": r["t_up"] * 1e6, "bytes_per_launch": up_bytes}
     else:
         P = cfg.T * cfg.top_k
         roofline = {"bound": "mfma", "achieved": 2.0 * P * cfg.K * cfg.N / r["t_up"] / 1e12,
                     "peak": PEAK_TFLOPS[cfg.dtype], "unit": "TFLOP/s",
-                    "kernel": "moe_up_kernel (gate/up GEMM + SwiGLU)", "launch_us": r["t_up"] * 1e6}
+                    "kernel": "moe_up_kernel_bf16 (gate/up GEMM + SwiGLU)", "launch_us": r["t_up"] * 1e6}
     roofline["frac"] = roofline["achieved"] / roofline["peak"]
     traffic, mfma_busy = recorded_traffic(cfg.name)  # the kernels do not depend on --split
     roofline["traffic"] = traffic
